@@ -43,8 +43,11 @@ def lookup_architecture(name: str) -> Architecture:
 
 def architecture_of(config_json: dict, where: str = "config.json") -> Architecture:
     archs = config_json.get("architectures")
+    if archs is None and isinstance(config_json.get("architecture"), str):     # a single name under the singular key
+        return lookup_architecture(config_json["architecture"])
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError(f"{where}: key 'architectures' must be a list naming the model class")
+        raise ConfigError(f"{where}: key 'architectures' must be a list naming the model class "
+                          f"(or 'architecture' its name)")
     return lookup_architecture(archs[0])
 
 

@@ -1,0 +1,284 @@
+// Attention whose keys and values have sizes of their own, with an optional sink: the cache
+// write with rotation of a part of each head, the plain attention kernel (one wave per (token,
+// head), both dtypes, any sizes), and a small per-head product.
+//
+// One kernel family serves two mixers.  Grouped attention with a key size Dk and a value size
+// Dv; and latent attention in its absorbed form: the per-head up-projection of the keys is
+// moved onto the query, so that every head scores against the one cached row [latent | rotated
+// part] (Dk = rank + rotated dims, one key/value head) and mixes the latents themselves
+// (Dv = rank); the per-head value up-projection follows the attention.
+//
+// The paged cache of a layer here is [pages][kv_heads][page_size * (Dk + Dv)]: the keys of a
+// (page, head) as [slot][Dk], then its values transposed as [Dv][slot] (`KvLayout`).
+//
+// softmax with a sink: the denominator holds one more term exp(sink_h), which has no key and
+// no value: p_j = exp(s_j - m) / (exp(sink_h - m) + sum_i exp(s_i - m)), m the maximum over
+// the scores and the sink.
+#include "attention_kv.h"
+
+using namespace hfee;
+
+namespace {
+
+// ---------------------------------------------------------------- rotation + cache write
+// One workgroup a token.  q is rotated in place; k (rotated) and v (blended, if asked) go
+// into the token's slot.  The rotated dims of a head are [rot_off, rot_off + 2 * half), pairs
+// (i, i + half); cos/sin tables [positions][half] carry the amplitude.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_write_kernel(
+    T* __restrict__ q, int64_t ldq, int num_heads, int q_dim, int q_rot_off,
+    const T* __restrict__ k, int64_t ldk, int k_rot_off, const T* __restrict__ v, int64_t ldv,
+    T* __restrict__ v_first, int v_first_mode, const T* __restrict__ v_mix,
+    const int* __restrict__ positions, const int* __restrict__ token_segment,
+    const int* __restrict__ block_tables, int bt_stride, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int half, T* __restrict__ cache, KvLayout lay) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const float* c = cos_t + (int64_t)pos * half;
+  const float* s = sin_t + (int64_t)pos * half;
+  if (q != nullptr) {
+    T* qr = q + (int64_t)t * ldq;
+    for (int e = threadIdx.x; e < num_heads * half; e += blockDim.x) {
+      const int h = e / half, i = e - h * half;
+      T* p = qr + (int64_t)h * q_dim + q_rot_off + i;
+      const float a = to_float<T>(p[0]), b = to_float<T>(p[half]);
+      p[0] = from_float<T>(a * c[i] - b * s[i]);
+      p[half] = from_float<T>(b * c[i] + a * s[i]);
+    }
+  }
+  if (k == nullptr) return;
+  const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
+  const int slot = pos & (lay.page_size - 1);
+  const T* kr = k + (int64_t)t * ldk;
+  for (int e = threadIdx.x; e < lay.kv_heads * lay.dk; e += blockDim.x) {
+    const int g = e / lay.dk, d = e - g * lay.dk;
+    const int i = d - k_rot_off;
+    float val;
+    if (i >= 0 && i < half) {
+      val = to_float<T>(kr[e]) * c[i] - to_float<T>(kr[e + half]) * s[i];
+    } else if (i >= half && i < 2 * half) {
+      val = to_float<T>(kr[e]) * c[i - half] + to_float<T>(kr[e - half]) * s[i - half];
+    } else {
+      val = to_float<T>(kr[e]);
+    }
+    cache[lay.key_offset(page, g, slot, d)] = finite_for_cache<T>(from_float<T>(val));
+  }
+  const T* vr = v + (int64_t)t * ldv;
+  const int vw = lay.kv_heads * lay.dv;
+  const float lam = v_first_mode == 2 ? to_float<T>(v_mix[0]) : 0.f;
+  for (int e = threadIdx.x; e < vw; e += blockDim.x) {
+    const int g = e / lay.dv, d = e - g * lay.dv;
+    T val = vr[e];
+    if (v_first_mode == 1) {
+      v_first[(int64_t)t * vw + e] = val;
+    } else if (v_first_mode == 2) {
+      val = from_float<T>((1.0f - lam) * to_float<T>(val) + lam * to_float<T>(v_first[(int64_t)t * vw + e]));
+    }
+    cache[lay.value_offset(page, g, slot, d)] = finite_for_cache<T>(val);
+  }
+}
+
+// ---------------------------------------------------------------- plain attention
+// Lane (j mod 64) owns key j, so which lane adds which term depends only on the key's
+// absolute position: a token's result does not change with the way the work was cut into
+// steps, with the batch around it or with page numbers.
+constexpr int kMaxDvPerLane = 8;      // value sizes up to 512
+
+template <typename T>
+__global__ __launch_bounds__(64) void attention_kv_plain_kernel(
+    T* __restrict__ out, int64_t ld_out, const T* __restrict__ q, int64_t ldq,
+    const T* __restrict__ cache, KvLayout lay, const int* __restrict__ positions,
+    const int* __restrict__ token_segment, const int* __restrict__ block_tables, int bt_stride,
+    int num_heads, float scale, const float* __restrict__ sinks) {
+  extern __shared__ float lds[];
+  const int dk = lay.dk, dv = lay.dv;
+  float* qs = lds;            // [dk]
+  float* es = lds + dk;       // [64]
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int kvh = h / (num_heads / lay.kv_heads);
+  const int pos = positions[t];
+  const int* bt = block_tables + (int64_t)token_segment[t] * bt_stride;
+
+  for (int d = lane; d < dk; d += 64) qs[d] = to_float<T>(q[(int64_t)t * ldq + (int64_t)h * dk + d]);
+  __syncthreads();
+
+  float m = -INFINITY;
+  for (int base = 0; base <= pos; base += 64) {
+    const int j = base + lane;
+    if (j <= pos) {
+      const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
+      float s = 0.f;
+      for (int d = 0; d < dk; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
+      m = fmaxf(m, s * scale);
+    }
+  }
+  m = wave_max(m);
+  const bool has_sink = sinks != nullptr;
+  const float sink = has_sink ? sinks[h] : 0.f;
+  if (has_sink) m = fmaxf(m, sink);
+
+  float lsum = 0.f;
+  float o[kMaxDvPerLane];
+#pragma unroll
+  for (int r = 0; r < kMaxDvPerLane; ++r) o[r] = 0.f;
+  for (int base = 0; base <= pos; base += 64) {
+    const int j = base + lane;
+    float e = 0.f;
+    if (j <= pos) {
+      const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), 0);
+      float s = 0.f;
+      for (int d = 0; d < dk; ++d) s = fmaf(qs[d], to_float<T>(kr[d]), s);
+      e = expf(s * scale - m);
+      lsum += e;
+    }
+    __syncthreads();
+    es[lane] = e;
+    __syncthreads();
+    const int je = min(base + 63, pos);
+    for (int jj = base; jj <= je; ++jj) {
+      const float w = es[jj - base];
+      const int page = bt[jj >> lay.page_shift], slot = jj & (lay.page_size - 1);
+#pragma unroll
+      for (int r = 0; r < kMaxDvPerLane; ++r) {
+        const int d = lane + 64 * r;
+        if (d < dv) o[r] = fmaf(w, to_float<T>(cache[lay.value_offset(page, kvh, slot, d)]), o[r]);
+      }
+    }
+  }
+  lsum = wave_sum(lsum);
+  if (has_sink) lsum += expf(sink - m);
+#pragma unroll
+  for (int r = 0; r < kMaxDvPerLane; ++r) {
+    const int d = lane + 64 * r;
+    if (d < dv) out[(int64_t)t * ld_out + (int64_t)h * dv + d] = from_float<T>(o[r] / lsum);
+  }
+}
+
+// ---------------------------------------------------------------- per-head product
+// out[t, h, o] = sum_i w[h][i][o] * x[t, h, i] for o < n_out (w stored [heads][n_in][n_out], so
+// that neighbouring threads read neighbouring weights), in ascending i; then `tail` elements
+// x[t, h, n_in ..] are copied behind them.  A workgroup takes one head and kTokens tokens.
+constexpr int kHeadLinearTokens = 8;
+
+template <typename T>
+__global__ __launch_bounds__(256) void head_linear_kernel(
+    T* __restrict__ out, int64_t ldo, int64_t out_head_stride, const T* __restrict__ x, int64_t ldx,
+    int64_t x_head_stride, const T* __restrict__ w, int n_in, int n_out, int tail, int n) {
+  extern __shared__ float xs[];      // [kTokens][n_in]
+  const int h = blockIdx.y, t0 = blockIdx.x * kHeadLinearTokens;
+  const int count = min(kHeadLinearTokens, n - t0);
+  for (int e = threadIdx.x; e < count * n_in; e += blockDim.x) {
+    const int r = e / n_in, i = e - r * n_in;
+    xs[e] = to_float<T>(x[(int64_t)(t0 + r) * ldx + (int64_t)h * x_head_stride + i]);
+  }
+  __syncthreads();
+  const T* wh = w + (int64_t)h * n_in * n_out;
+  for (int o = threadIdx.x; o < n_out; o += blockDim.x) {
+    float acc[kHeadLinearTokens];
+#pragma unroll
+    for (int r = 0; r < kHeadLinearTokens; ++r) acc[r] = 0.f;
+    for (int i = 0; i < n_in; ++i) {
+      const float wv = to_float<T>(wh[(int64_t)i * n_out + o]);
+#pragma unroll
+      for (int r = 0; r < kHeadLinearTokens; ++r) acc[r] = fmaf(wv, xs[r * n_in + i], acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < kHeadLinearTokens; ++r)
+      if (r < count) out[(int64_t)(t0 + r) * ldo + (int64_t)h * out_head_stride + o] = from_float<T>(acc[r]);
+  }
+  for (int e = threadIdx.x; e < count * tail; e += blockDim.x) {
+    const int r = e / tail, i = e - r * tail;
+    out[(int64_t)(t0 + r) * ldo + (int64_t)h * out_head_stride + n_out + i] =
+        x[(int64_t)(t0 + r) * ldx + (int64_t)h * x_head_stride + n_in + i];
+  }
+}
+
+}  // namespace
+
+HFEE_API int hfee_kv_write(void* q, int64_t ldq, int num_heads, int q_dim, int q_rot_off, const void* k, int64_t ldk,
+                           int k_rot_off, const void* v, int64_t ldv, void* v_first, int v_first_mode,
+                           const void* v_mix, int dtype, const int* positions, const int* token_segment,
+                           const int* block_tables, int bt_stride, const float* cos_t, const float* sin_t, int half,
+                           int table_positions, int max_position, void* cache, int kv_heads, int dk, int dv,
+                           int page_size, int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0, "kv_write: bad token count");
+  if (n == 0) return 0;
+  HFEE_REQUIRE(q != nullptr || k != nullptr, "kv_write: nothing to do");
+  HFEE_REQUIRE(half >= 0 && (half == 0 || (cos_t != nullptr && sin_t != nullptr)), "kv_write: rotation tables missing");
+  HFEE_REQUIRE(half == 0 || max_position < table_positions,
+               "kv_write: position %d is beyond the rotation tables of %d positions", max_position, table_positions);
+  HFEE_REQUIRE(q == nullptr || (q_rot_off >= 0 && q_rot_off + 2 * half <= q_dim && ldq >= (int64_t)num_heads * q_dim),
+               "kv_write: the rotated dims do not fit the query heads");
+  HFEE_REQUIRE(v_first_mode >= 0 && v_first_mode <= 2 && (v_first_mode == 0 || v_first != nullptr) &&
+               (v_first_mode != 2 || v_mix != nullptr), "kv_write: value blending needs its buffers");
+  KvLayout lay;
+  if (k != nullptr) {
+    HFEE_REQUIRE(v != nullptr && cache != nullptr && token_segment != nullptr && block_tables != nullptr,
+                 "kv_write: k, v, the cache and the block tables come together");
+    if (make_kv_layout(&lay, kv_heads, dk, dv, page_size)) return 1;
+    HFEE_REQUIRE(k_rot_off >= 0 && k_rot_off + 2 * half <= dk, "kv_write: the rotated dims do not fit the key heads");
+    HFEE_REQUIRE(ldk >= (int64_t)kv_heads * dk && ldv >= (int64_t)kv_heads * dv, "kv_write: k/v rows too short");
+  } else {
+    lay = KvLayout{};
+  }
+#define LAUNCH(T)                                                                                                    \
+  kv_write_kernel<T><<<n, 256, 0, stream>>>((T*)q, ldq, num_heads, q_dim, q_rot_off, (const T*)k, ldk, k_rot_off,    \
+      (const T*)v, ldv, (T*)v_first, v_first_mode, (const T*)v_mix, positions, token_segment, block_tables,          \
+      bt_stride, cos_t, sin_t, half, (T*)cache, lay)
+  if (dtype == 0) LAUNCH(float);
+  else if (dtype == 1) LAUNCH(bf16_t);
+  else return fail("kv_write: unknown dtype %d", dtype);
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("kv_write");
+  return 0;
+}
+
+HFEE_API int hfee_attention_kv_plain(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
+                                     int dtype, const int* positions, const int* token_segment,
+                                     const int* block_tables, int bt_stride, int num_heads, int kv_heads, int dk,
+                                     int dv, int page_size, float scale, const float* sinks, int n,
+                                     hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0, "attention_kv_plain: bad token count");
+  if (n == 0) return 0;
+  HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
+               "attention_kv_plain: %d heads are not a multiple of %d kv heads", num_heads, kv_heads);
+  HFEE_REQUIRE(dk >= 1 && dk <= 4096 && dv >= 1 && dv <= 64 * kMaxDvPerLane,
+               "attention_kv_plain: key size %d or value size %d is out of range", dk, dv);
+  HFEE_REQUIRE(num_heads <= 65535, "attention_kv_plain: too many heads");
+  HFEE_REQUIRE(ldq >= (int64_t)num_heads * dk && ld_out >= (int64_t)num_heads * dv, "attention_kv_plain: q/out row too short");
+  KvLayout lay;
+  if (make_kv_layout(&lay, kv_heads, dk, dv, page_size)) return 1;
+  dim3 grid(n, num_heads);
+  const size_t lds = (dk + 64) * sizeof(float);
+  if (dtype == 0)
+    attention_kv_plain_kernel<float><<<grid, 64, lds, stream>>>((float*)out, ld_out, (const float*)q, ldq,
+        (const float*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks);
+  else if (dtype == 1)
+    attention_kv_plain_kernel<bf16_t><<<grid, 64, lds, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
+        (const bf16_t*)cache, lay, positions, token_segment, block_tables, bt_stride, num_heads, scale, sinks);
+  else
+    return fail("attention_kv_plain: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("attention_kv_plain");
+  return 0;
+}
+
+HFEE_API int hfee_head_linear(void* out, int64_t ldo, int64_t out_head_stride, const void* x, int64_t ldx,
+                              int64_t x_head_stride, const void* w, int dtype, int heads, int n_in, int n_out,
+                              int tail, int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && heads > 0 && n_in > 0 && n_out > 0 && tail >= 0, "head_linear: bad sizes");
+  if (n == 0) return 0;
+  HFEE_REQUIRE(heads <= 65535 && n_in <= 2048, "head_linear: at most 65535 heads and 2048 inputs a head");
+  HFEE_REQUIRE(x_head_stride >= n_in + tail && out_head_stride >= n_out + tail, "head_linear: heads overlap");
+  dim3 grid((n + kHeadLinearTokens - 1) / kHeadLinearTokens, heads);
+  const size_t lds = (size_t)kHeadLinearTokens * n_in * sizeof(float);
+  if (dtype == 0)
+    head_linear_kernel<float><<<grid, 256, lds, stream>>>((float*)out, ldo, out_head_stride, (const float*)x, ldx,
+        x_head_stride, (const float*)w, n_in, n_out, tail, n);
+  else if (dtype == 1)
+    head_linear_kernel<bf16_t><<<grid, 256, lds, stream>>>((bf16_t*)out, ldo, out_head_stride, (const bf16_t*)x, ldx,
+        x_head_stride, (const bf16_t*)w, n_in, n_out, tail, n);
+  else
+    return fail("head_linear: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("head_linear");
+  return 0;
+}

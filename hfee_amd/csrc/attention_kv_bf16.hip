@@ -1,0 +1,268 @@
+// Matrix-core attention over the paged cache for keys of HFEE_DK and values of HFEE_DV dims
+// (multiples of 16, compiled per pair), with an optional sink; bfloat16 operands, float32
+// scores, weights and sums.  The cache layout is `KvLayout` (attention_kv.h).
+//
+// A wave owns 16 query rows and walks tiles of 32 keys: S^T = K Q^T (the keys are the row
+// operand: a lane loads eight dims of one key, 16 bytes), then O^T += V^T P^T with the
+// weights as they stand in the score registers (the k index of a matrix instruction is only a
+// label shared by both operands: label 8g + e of lane group g means key 4g + e of the tile's
+// first 16 keys for e < 4 and key 4g + e - 4 of its second 16 otherwise, so a lane's eight
+// values of a value column are two loads of 8 bytes from the transposed values).
+//
+// Two meanings of the 16 rows (`mode`):
+//   0  a portion of a prompt: 16 consecutive tokens of one sequence, one head a wave;
+//   1  a single token: up to 16 query heads that share a key/value head; the keys may be
+//      split over several waves, whose partial results a second kernel joins.
+// The sink joins the denominator once, at the very end.
+#include "attention_kv.h"
+
+#ifndef HFEE_DK
+#error "compile with -DHFEE_DK=<key size> -DHFEE_DV=<value size>"
+#endif
+
+using namespace hfee;
+
+namespace {
+
+constexpr int DK = HFEE_DK, DV = HFEE_DV;
+static_assert(DK % 16 == 0 && DV % 16 == 0 && DK >= 16 && DV >= 16, "key and value sizes are multiples of 16");
+constexpr int KSTEPS = (DK + 31) / 32;     // steps of 32 dims (the last may be half empty)
+constexpr int VBLOCKS = DV / 16;
+constexpr float kLog2e = 1.4426950408889634f;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+union Operand {
+  bf16x8 v;
+  u32x4 u;
+  u32x2 h[2];
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  return (uint32_t)float_to_bf16(a) | ((uint32_t)float_to_bf16(b) << 16);
+}
+
+// partial results of a split: [item][head][split][4 + DV] float32: maximum (base 2), sum, two unused, O
+constexpr int kPartial = 4 + DV;
+
+template <int MODE>
+__global__ __launch_bounds__(256) void attention_kv_kernel(
+    bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
+    const bf16_t* __restrict__ cache, KvLayout lay, const int* __restrict__ items, int num_items,
+    const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2,
+    const float* __restrict__ sinks, float* __restrict__ partial, int splits) {
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+  const int hpg = num_heads / lay.kv_heads;
+  const int groups16 = (hpg + 15) / 16;
+  const int units = MODE == 0 ? num_heads : lay.kv_heads * groups16;
+  const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (wave >= (int64_t)num_items * splits * units) return;
+  const int unit = (int)(wave % units);
+  const int split = (int)((wave / units) % splits);
+  const int item = (int)(wave / ((int64_t)units * splits));
+  const int row0 = items[item * 4 + 0], rows = items[item * 4 + 1], pos0 = items[item * 4 + 2];
+  const int* bt = block_tables + (int64_t)items[item * 4 + 3] * bt_stride;
+
+  int token, head, pos, kvh;
+  bool valid;
+  if (MODE == 0) {
+    const int rr = min(r, rows - 1);
+    token = row0 + rr; pos = pos0 + rr; head = unit; kvh = head / hpg; valid = r < rows;
+  } else {
+    kvh = unit / groups16;
+    const int in_group = (unit % groups16) * 16 + r;
+    valid = in_group < hpg;
+    token = row0; pos = pos0; head = kvh * hpg + min(in_group, hpg - 1);
+  }
+  const int max_pos = MODE == 0 ? pos0 + rows - 1 : pos0;
+
+  // the queries as the column operand: lane (r, g) holds dims 8g .. 8g+7 of every step of row r
+  Operand qop[KSTEPS];
+  {
+    const bf16_t* qr = q + (int64_t)token * ldq + (int64_t)head * DK + g * 8;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      if (s * 32 + g * 8 < DK) qop[s].u = *reinterpret_cast<const u32x4*>(qr + s * 32);
+      else qop[s].u = u32x4{0, 0, 0, 0};
+    }
+  }
+
+  f32x4 acc[VBLOCKS];
+#pragma unroll
+  for (int b = 0; b < VBLOCKS; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+
+  const int ntiles = (max_pos >> 5) + 1;
+  const int per_split = (ntiles + splits - 1) / splits;
+  const int tile_begin = split * per_split, tile_end = min(ntiles, tile_begin + per_split);
+  const int last_block = max_pos >> lay.page_shift;
+  const int slot_mask = lay.page_size - 1;
+
+  for (int tile = tile_begin; tile < tile_end; ++tile) {
+    const int j0 = tile << 5;
+    f32x4 s[2];
+    const bf16_t* vbase[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const int jb = j0 + b * 16;
+      const int page = bt[min(jb >> lay.page_shift, last_block)];
+      const int slot0 = jb & slot_mask;
+      const bf16_t* kr = cache + lay.key_offset(page, kvh, slot0 + r, g * 8);
+      vbase[b] = cache + lay.values_of(page, kvh) + slot0 + g * 4;
+      s[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < KSTEPS; ++st) {
+        Operand kop;
+        if (st * 32 + g * 8 < DK) kop.u = *reinterpret_cast<const u32x4*>(kr + st * 32);
+        else kop.u = u32x4{0, 0, 0, 0};
+        s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qop[st].v, s[b], 0, 0, 0);
+      }
+    }
+    // scores of query r (this lane's column) against keys j0 + 16 b + 4 g + i
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = j0 + b * 16 + g * 4 + i;
+        const float v = key <= pos ? s[b][i] * scale_log2 : -INFINITY;
+        s[b][i] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = exp2f(m - m_use);
+    m = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = exp2f(s[b][i] - m_use);
+        s[b][i] = p;
+        psum += p;
+      }
+    lsum = lsum * alpha + psum;
+    Operand pop;
+    pop.u = u32x4{pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]), pack_bf16(s[1][0], s[1][1]),
+                  pack_bf16(s[1][2], s[1][3])};
+#pragma unroll
+    for (int vb = 0; vb < VBLOCKS; ++vb) {
+      Operand vop;
+      const int64_t column = (int64_t)(vb * 16 + r) * lay.page_size;
+      vop.h[0] = *reinterpret_cast<const u32x2*>(vbase[0] + column);
+      vop.h[1] = *reinterpret_cast<const u32x2*>(vbase[1] + column);
+      acc[vb] = acc[vb] * alpha;
+      acc[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop.v, acc[vb], 0, 0, 0);
+    }
+  }
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+
+  if (splits == 1) {
+    if (sinks != nullptr) {
+      const float sk = sinks[head] * kLog2e;
+      const float m_all = fmaxf(m, sk);
+      const float a = exp2f(m - m_all);
+      lsum = lsum * a + exp2f(sk - m_all);
+#pragma unroll
+      for (int vb = 0; vb < VBLOCKS; ++vb) acc[vb] = acc[vb] * a;
+    }
+    if (!valid) return;
+    const float inv = 1.0f / lsum;
+    bf16_t* orow = out + (int64_t)token * ld_out + (int64_t)head * DV + g * 4;
+#pragma unroll
+    for (int vb = 0; vb < VBLOCKS; ++vb) {
+      const u32x2 w = {pack_bf16(acc[vb][0] * inv, acc[vb][1] * inv), pack_bf16(acc[vb][2] * inv, acc[vb][3] * inv)};
+      *reinterpret_cast<u32x2*>(orow + vb * 16) = w;
+    }
+    return;
+  }
+  if (!valid) return;
+  float* pr = partial + (((int64_t)item * num_heads + head) * splits + split) * kPartial;
+  if (g == 0) {
+    pr[0] = m;
+    pr[1] = lsum;
+  }
+#pragma unroll
+  for (int vb = 0; vb < VBLOCKS; ++vb)
+    *reinterpret_cast<f32x4*>(pr + 4 + vb * 16 + g * 4) = acc[vb];
+}
+
+// joins the splits of a single token's heads: one wave per (item, head), lanes over the value dims
+__global__ __launch_bounds__(64) void attention_kv_join_kernel(
+    bf16_t* __restrict__ out, int64_t ld_out, const int* __restrict__ items, const float* __restrict__ partial,
+    int splits, int num_heads, const float* __restrict__ sinks) {
+  const int item = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const float* pr = partial + ((int64_t)item * num_heads + head) * splits * kPartial;
+  float m = sinks != nullptr ? sinks[head] * kLog2e : -INFINITY;
+  for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, pr[sp * kPartial]);
+  float lsum = sinks != nullptr ? exp2f(sinks[head] * kLog2e - m) : 0.f;
+  for (int sp = 0; sp < splits; ++sp) lsum += pr[sp * kPartial + 1] * exp2f(pr[sp * kPartial] - m);
+  const int token = items[item * 4];
+  for (int d = lane; d < DV; d += 64) {
+    float o = 0.f;
+    for (int sp = 0; sp < splits; ++sp) o += pr[sp * kPartial + 4 + d] * exp2f(pr[sp * kPartial] - m);
+    out[(int64_t)token * ld_out + (int64_t)head * DV + d] = float_to_bf16(o / lsum);
+  }
+}
+
+}  // namespace
+
+HFEE_DEFINE_LAST_ERROR
+
+HFEE_API int hfee_attention_kv_bf16_dk() { return DK; }
+HFEE_API int hfee_attention_kv_bf16_dv() { return DV; }
+
+// float32 words of `partial` that `splits` > 1 need for `num_items` single tokens
+HFEE_API int64_t hfee_attention_kv_bf16_partial(int num_items, int num_heads, int splits) {
+  return splits > 1 ? (int64_t)num_items * num_heads * splits * kPartial : 0;
+}
+
+// items: [num_items][4] int32 on the device: first row, rows (1..16; 1 in mode 1), first
+// position, block-table row.
+HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
+                                    const int* items, int num_items, int mode, const int* block_tables,
+                                    int bt_stride, int num_heads, int kv_heads, int page_size, float scale,
+                                    const float* sinks, float* partial, int64_t partial_words, int splits,
+                                    hipStream_t stream) {
+  HFEE_REQUIRE(num_items >= 0, "attention_kv_bf16: bad item count");
+  if (num_items == 0) return 0;
+  HFEE_REQUIRE(mode == 0 || mode == 1, "attention_kv_bf16: mode is 0 (portions) or 1 (single tokens)");
+  HFEE_REQUIRE(num_heads > 0 && kv_heads > 0 && num_heads % kv_heads == 0,
+               "attention_kv_bf16: %d heads are not a multiple of %d kv heads", num_heads, kv_heads);
+  HFEE_REQUIRE(num_heads <= 65535, "attention_kv_bf16: too many heads");
+  HFEE_REQUIRE(ldq >= (int64_t)num_heads * DK && ld_out >= (int64_t)num_heads * DV, "attention_kv_bf16: q/out row too short");
+  HFEE_REQUIRE(ldq % 8 == 0 && ld_out % 4 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)out % 8 == 0 &&
+               (uintptr_t)cache % 16 == 0, "attention_kv_bf16: q, out and the cache must be aligned for vector access");
+  HFEE_REQUIRE(splits >= 1 && (splits == 1 || mode == 1), "attention_kv_bf16: only single tokens split their keys");
+  HFEE_REQUIRE(splits == 1 || (partial != nullptr &&
+               partial_words >= hfee_attention_kv_bf16_partial(num_items, num_heads, splits)),
+               "attention_kv_bf16: the partial results need more room");
+  KvLayout lay;
+  if (make_kv_layout(&lay, kv_heads, DK, DV, page_size)) return 1;
+  const int hpg = num_heads / kv_heads;
+  const int64_t units = mode == 0 ? num_heads : (int64_t)kv_heads * ((hpg + 15) / 16);
+  const int64_t waves = (int64_t)num_items * splits * units;
+  const int64_t blocks = (waves + 3) / 4;
+  HFEE_REQUIRE(blocks <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
+  const float scale_log2 = scale * kLog2e;
+  if (mode == 0)
+    attention_kv_kernel<0><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
+        (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scale_log2, sinks, partial, 1);
+  else
+    attention_kv_kernel<1><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
+        (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scale_log2, sinks, partial, splits);
+  HFEE_CHECK_LAUNCH("attention_kv_bf16");
+  if (splits > 1) {
+    attention_kv_join_kernel<<<dim3(num_items, num_heads), 64, 0, stream>>>((bf16_t*)out, ld_out, items, partial,
+                                                                            splits, num_heads, sinks);
+    HFEE_CHECK_LAUNCH("attention_kv_bf16 join");
+  }
+  return 0;
+}

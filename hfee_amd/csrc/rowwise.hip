@@ -1,0 +1,168 @@
+// Row-wise steps of blocks that norm a sub-layer's output before they add it to the residual
+// stream, and of feed-forwards with biases:
+//
+//   norm_add:      x[r] += (y[r] + bias) / sqrt(mean((y[r] + bias)^2) + eps) * w,   and, if asked, in
+//                  the same launch the norm of the new row for the sub-layer that follows:
+//                  next[r] = x[r] / sqrt(mean(x[r]^2) + eps2) * w2
+//   bias_act:      out = act(in + bias)
+//   rmsnorm_cols:  a norm over a block of columns of rows in the engine's dtype (a latent's norm)
+//
+// All sums in float32, one workgroup a row, a fixed order of additions.
+#include "common.h"
+
+using namespace hfee;
+
+namespace {
+
+enum { ACT_NONE = 0, ACT_RELU2 = 1, ACT_RELU = 2, ACT_GELU_TANH = 3, ACT_SILU = 4 };
+
+__device__ __forceinline__ float activate(float z, int act) {
+  switch (act) {
+    case ACT_RELU2: { const float r = fmaxf(z, 0.f); return r * r; }
+    case ACT_RELU: return fmaxf(z, 0.f);
+    case ACT_GELU_TANH: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    case ACT_SILU: return z / (1.0f + expf(-z));
+    default: return z;
+  }
+}
+
+template <typename TW>
+__device__ __forceinline__ float weight_at(const TW* w, int j, float offset) { return offset + to_float<TW>(w[j]); }
+
+// y: float32 [n, d]; bias: engine dtype or null; w, w2: norm weights (TW), used as (offset + w).
+template <typename TY, typename TB, typename TW, typename TN>
+__global__ __launch_bounds__(256) void norm_add_kernel(
+    float* __restrict__ x, const TY* __restrict__ y, const TB* __restrict__ bias, const TW* __restrict__ w, float offset,
+    float eps, TN* __restrict__ next, const TW* __restrict__ w2, float eps2, int d) {
+  __shared__ float scratch[16];
+  const int64_t r = blockIdx.x;
+  const TY* yr = y + r * d;
+  float* xr = x + r * d;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) {
+    const float v = to_float<TY>(yr[j]) + (bias ? to_float<TB>(bias[j]) : 0.f);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  float ss2 = 0.f;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) {
+    const float v = to_float<TY>(yr[j]) + (bias ? to_float<TB>(bias[j]) : 0.f);
+    const float nx = xr[j] + v * inv * weight_at<TW>(w, j, offset);
+    xr[j] = nx;
+    ss2 = fmaf(nx, nx, ss2);
+  }
+  if (next == nullptr) return;
+  ss2 = block_sum(ss2, scratch);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)d + eps2);
+  TN* nr = next + r * d;
+  for (int j = threadIdx.x; j < d; j += blockDim.x)      // (a thread reads back what it wrote itself)
+    nr[j] = from_float<TN>(xr[j] * inv2 * weight_at<TW>(w2, j, offset));
+}
+
+template <typename T>
+__global__ void bias_act_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ in, int64_t ldi,
+                                const T* __restrict__ bias, int width, int act) {
+  const int64_t row = blockIdx.y;
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= width) return;
+  const float z = to_float<T>(in[row * ldi + j]) + (bias ? to_float<T>(bias[j]) : 0.f);
+  out[row * ldo + j] = from_float<T>(activate(z, act));
+}
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void rmsnorm_cols_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ x,
+                                                           int64_t ldx, const TW* __restrict__ w, float offset,
+                                                           float eps, int width) {
+  __shared__ float scratch[16];
+  const int64_t r = blockIdx.x;
+  const T* xr = x + r * ldx;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    const float v = to_float<T>(xr[j]);
+    ss = fmaf(v, v, ss);
+  }
+  ss = block_sum(ss, scratch);       // (its barriers stand between every read of the row and the writes: in place is fine)
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  T* orow = out + r * ldo;
+  for (int j = threadIdx.x; j < width; j += blockDim.x)
+    orow[j] = from_float<T>(to_float<T>(xr[j]) * inv * weight_at<TW>(w, j, offset));
+}
+
+}  // namespace
+
+// y_dtype / bias_dtype / w_dtype / next_dtype: 0 float32, 1 bfloat16.
+HFEE_API int hfee_norm_add(float* x, const void* y, int y_dtype, const void* bias, int bias_dtype, const void* w,
+                           int w_dtype, float offset, float eps, void* next, int next_dtype, const void* w2,
+                           float eps2, int n, int d, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && d > 0, "norm_add: bad sizes n=%d d=%d", n, d);
+  HFEE_REQUIRE(eps >= 0.f && eps2 >= 0.f, "norm_add: eps must not be negative");
+  HFEE_REQUIRE(next == nullptr || w2 != nullptr, "norm_add: the following norm needs its weight");
+  if (n == 0) return 0;
+  const int code = (y_dtype & 1) | ((bias_dtype & 1) << 1) | ((w_dtype & 1) << 2) | ((next_dtype & 1) << 3);
+#define CASE(c, TY, TB, TW, TN)                                                                                      \
+  case c:                                                                                                            \
+    norm_add_kernel<TY, TB, TW, TN><<<n, 256, 0, stream>>>(x, (const TY*)y, (const TB*)bias, (const TW*)w, offset,   \
+        eps, (TN*)next, (const TW*)w2, eps2, d);                                                                     \
+    break
+  switch (code) {
+    CASE(0, float, float, float, float);
+    CASE(1, bf16_t, float, float, float);
+    CASE(2, float, bf16_t, float, float);
+    CASE(3, bf16_t, bf16_t, float, float);
+    CASE(4, float, float, bf16_t, float);
+    CASE(5, bf16_t, float, bf16_t, float);
+    CASE(6, float, bf16_t, bf16_t, float);
+    CASE(7, bf16_t, bf16_t, bf16_t, float);
+    CASE(8, float, float, float, bf16_t);
+    CASE(9, bf16_t, float, float, bf16_t);
+    CASE(10, float, bf16_t, float, bf16_t);
+    CASE(11, bf16_t, bf16_t, float, bf16_t);
+    CASE(12, float, float, bf16_t, bf16_t);
+    CASE(13, bf16_t, float, bf16_t, bf16_t);
+    CASE(14, float, bf16_t, bf16_t, bf16_t);
+    CASE(15, bf16_t, bf16_t, bf16_t, bf16_t);
+  }
+#undef CASE
+  HFEE_CHECK_LAUNCH("norm_add");
+  return 0;
+}
+
+HFEE_API int hfee_bias_act(void* out, int64_t ldo, const void* in, int64_t ldi, const void* bias, int dtype, int n,
+                           int width, int act, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && width > 0, "bias_act: bad sizes");
+  HFEE_REQUIRE(act >= ACT_NONE && act <= ACT_SILU, "bias_act: unknown activation %d", act);
+  HFEE_REQUIRE(n <= 65535 * 32, "bias_act: too many rows");
+  if (n == 0) return 0;
+  for (int r0 = 0; r0 < n; r0 += 65535) {
+    const int rows = n - r0 < 65535 ? n - r0 : 65535;
+    dim3 grid((width + 255) / 256, rows);
+    if (dtype == 0)
+      bias_act_kernel<float><<<grid, 256, 0, stream>>>((float*)out + (int64_t)r0 * ldo, ldo, (const float*)in + (int64_t)r0 * ldi,
+                                                        ldi, (const float*)bias, width, act);
+    else if (dtype == 1)
+      bias_act_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out + (int64_t)r0 * ldo, ldo, (const bf16_t*)in + (int64_t)r0 * ldi,
+                                                         ldi, (const bf16_t*)bias, width, act);
+    else
+      return fail("bias_act: unknown dtype %d", dtype);
+  }
+  HFEE_CHECK_LAUNCH("bias_act");
+  return 0;
+}
+
+HFEE_API int hfee_rmsnorm_cols(void* out, int64_t ldo, const void* x, int64_t ldx, int dtype, const void* w, int w_dtype,
+                               float offset, float eps, int n, int width, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && width > 0, "rmsnorm_cols: bad sizes");
+  HFEE_REQUIRE(eps >= 0.f, "rmsnorm_cols: eps must not be negative");
+  if (n == 0) return 0;
+#define LAUNCH(T, TW)                                                                                                \
+  rmsnorm_cols_kernel<T, TW><<<n, 256, 0, stream>>>((T*)out, ldo, (const T*)x, ldx, (const TW*)w, offset, eps, width)
+  if (dtype == 0 && w_dtype == 0) LAUNCH(float, float);
+  else if (dtype == 0 && w_dtype == 1) LAUNCH(float, bf16_t);
+  else if (dtype == 1 && w_dtype == 0) LAUNCH(bf16_t, float);
+  else if (dtype == 1 && w_dtype == 1) LAUNCH(bf16_t, bf16_t);
+  else return fail("rmsnorm_cols: unknown dtypes");
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("rmsnorm_cols");
+  return 0;
+}

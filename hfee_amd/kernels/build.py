@@ -3,7 +3,9 @@
 Two kinds of library:
   * `core`: every kernel whose sizes are run-time arguments;
   * `attention_bf16_hd<N>`: the matrix-core attention kernels, compiled for one head
-    size each, on demand (a model compiles only the head size it has).
+    size each, on demand (a model compiles only the head size it has);
+  * `attention_kv_bf16_k<Dk>_v<Dv>`: the matrix-core attention for keys and values of
+    different sizes, compiled per pair of sizes, on demand.
 Libraries are built in-tree (hfee_amd/_lib); if that folder cannot be written, in a
 per-user folder under the system's temporary directory; $HFEE_BUILD_DIR, if set, comes
 before both.  A library is rebuilt when its sources or flags no longer match the stamp
@@ -31,9 +33,11 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fvisibility=h
          "-Wno-unused-command-line-argument"]
 
 CORE_SOURCES = ["elementwise.hip", "gemm_f32.hip", "attention_ref.hip", "gemm_bf16.hip", "gemm_skinny.hip",
-                "sampling.hip", "random_fill.hip", "yardstick.hip"]
+                "sampling.hip", "random_fill.hip", "yardstick.hip", "attention_kv.hip", "rowwise.hip"]
 ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
+ATTENTION_KV_SOURCE = "attention_kv_bf16.hip"      # compiled per (key size, value size)
+ATTENTION_KV_MOST = (1024, 512)
 
 
 class BuildError(RuntimeError):
@@ -98,6 +102,15 @@ def library_spec(name: str):
             raise BuildError(f"attention kernels exist for head sizes {HEAD_DIMS[0]}..{HEAD_DIMS[-1]} "
                              f"in steps of 16, not {hd}")
         return [ATTENTION_SOURCE], [f"-DHFEE_HEAD_DIM={hd}"]
+    if name.startswith("attention_kv_bf16_k"):
+        try:
+            dk, dv = (int(n) for n in name[len("attention_kv_bf16_k"):].split("_v"))
+        except ValueError:
+            raise BuildError(f"unknown kernel library {name!r}") from None
+        if dk % 16 or dv % 16 or not 16 <= dk <= ATTENTION_KV_MOST[0] or not 16 <= dv <= ATTENTION_KV_MOST[1]:
+            raise BuildError(f"the attention kernels for keys and values of different sizes take multiples of 16 up to "
+                             f"{ATTENTION_KV_MOST}, not ({dk}, {dv})")
+        return [ATTENTION_KV_SOURCE], [f"-DHFEE_DK={dk}", f"-DHFEE_DV={dv}"]
     raise BuildError(f"unknown kernel library {name!r}")
 
 

@@ -47,6 +47,18 @@ _CORE_SIGNATURES = {
     "hfee_random_fill": [P, I, L, U64, I, D, L, P],
     "hfee_read_stream": [P, L, P, I, I, P],
     "hfee_mfma_loop": [P, I, I, P],
+    "hfee_kv_write": [P, L, I, I, I, P, L, I, P, L, P, I, P, I, P, P, P, I, P, P, I, I, I, P, I, I, I, I, I, P],
+    "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, P],
+    "hfee_head_linear": [P, L, L, P, L, L, P, I, I, I, I, I, I, P],
+    "hfee_norm_add": [P, P, I, P, I, P, I, F, F, P, I, P, F, I, I, P],
+    "hfee_bias_act": [P, L, P, L, P, I, I, I, I, P],
+    "hfee_rmsnorm_cols": [P, L, P, L, I, P, I, F, F, I, I, P],
+}
+
+_ATTENTION_KV_SIGNATURES = {
+    "hfee_attention_kv_bf16_dk": [],
+    "hfee_attention_kv_bf16_dv": [],
+    "hfee_attention_kv_bf16": [P, L, P, L, P, P, I, I, P, I, I, I, I, F, P, P, L, I, P],
 }
 
 _ATTENTION_SIGNATURES = {
@@ -98,7 +110,8 @@ def load(name: str) -> Library:
                 path = build.build_library(name)
             except build.BuildError as e:
                 raise KernelLibraryError(f"the HIP kernel library '{name}' is not available: {e}") from None
-            sigs = _CORE_SIGNATURES if name == "core" else _ATTENTION_SIGNATURES
+            sigs = (_CORE_SIGNATURES if name == "core" else
+                    _ATTENTION_KV_SIGNATURES if name.startswith("attention_kv_bf16") else _ATTENTION_SIGNATURES)
             lib = _loaded[name] = Library(name, path, sigs)
         return lib
 
@@ -112,3 +125,11 @@ def attention_bf16(head_dim: int) -> Library:
         raise KernelError(f"the bfloat16 attention kernels take head sizes 16..256 in steps of 16, "
                           f"not {head_dim}")
     return load(f"attention_bf16_hd{head_dim}")
+
+
+def attention_kv_bf16(dk: int, dv: int) -> Library:
+    """The matrix-core attention for keys of dk and values of dv dims (multiples of 16)."""
+    if dk % 16 or dv % 16 or dk < 16 or dv < 16:
+        raise KernelError(f"the bfloat16 attention kernels for keys and values of different sizes take multiples "
+                          f"of 16, not ({dk}, {dv})")
+    return load(f"attention_kv_bf16_k{dk}_v{dv}")

@@ -787,3 +787,186 @@ def _qkv_rows(out, x, weight, q):
     lib.core().call("hfee_gemm_qkv_rows", _ptr(out), ldc, _ptr(x), lda, _ptr(weight), ldw, M, N, K,
                     _ptr(q["positions"]), _ptr(q.get("token_segment")), _ptr(bt), 0 if bt is None else bt.stride(0),
                     _ptr(cos), _ptr(sin), half, table_positions, _ptr(cache), H, KV, hd, ps, _stream())
+
+
+# ------------------------------- attention with keys and values of sizes of their own, and a sink
+
+def _kv_cache(cache_layer, kv_heads, dk, dv, page_size, what):
+    _check(cache_layer.is_contiguous() and cache_layer.dim() == 3 and
+           tuple(cache_layer.shape[1:]) == (kv_heads, page_size * (dk + dv)),
+           f"{what}: the cache layer must be [pages, kv_heads, page_size * (key size + value size)]")
+
+
+def kv_write(q, k, v, positions, token_segment, block_tables, cos, sin, cache_layer, num_heads: int, kv_heads: int,
+             q_dim: int, dk: int, dv: int, page_size: int, max_position: int, q_rot_offset: int = 0,
+             k_rot_offset: int = 0, v_first=None, v_first_mode: int = 0, v_mix=None):
+    """Rotates q in place and writes k (rotated) and v into the pages of `cache_layer`
+    ([pages, kv_heads, page_size * (dk + dv)]: keys [slot][dk], then values [dv][slot]).
+    q: [n, num_heads * q_dim] or None; k: [n, kv_heads * dk], v: [n, kv_heads * dv] or both None.
+    The rotated dims of a q head are [q_rot_offset, q_rot_offset + 2 * half), of a k head
+    [k_rot_offset, ...), pairs (i, i + half); cos/sin: float32 [positions, half] or None.
+    v_first_mode 1: v is also copied to v_first ([n, kv_heads * dv], contiguous); 2: what is written
+    is (1 - v_mix) v + v_mix v_first, v_mix a tensor of one element on the device."""
+    _gpu(q, k, v, positions, cos, sin, cache_layer, v_first, v_mix)
+    some = q if q is not None else k
+    _check(some is not None, "kv_write: nothing to do")
+    n = some.shape[0]
+    ldq = ldk = ldv = 0
+    if q is not None:
+        nq, wq, ldq = _rows2d(q, "kv_write q")
+        _check(nq == n and wq == num_heads * q_dim, "kv_write: q shape")
+    if k is not None:
+        _check(v is not None and cache_layer is not None, "kv_write: k, v and the cache come together")
+        nk, wk, ldk = _rows2d(k, "kv_write k")
+        nv, wv, ldv = _rows2d(v, "kv_write v")
+        _check(nk == n and nv == n and wk == kv_heads * dk and wv == kv_heads * dv, "kv_write: k/v shape")
+        _check(k.dtype == v.dtype == cache_layer.dtype and (q is None or q.dtype == k.dtype), "kv_write: dtype mismatch")
+        _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "kv_write")
+        _i32(token_segment, "kv_write token_segment", n)
+        _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+               "kv_write: block tables")
+        if v_first_mode:
+            _check(v_first is not None and v_first.is_contiguous() and v_first.dtype == v.dtype
+                   and tuple(v_first.shape) == (n, kv_heads * dv), "kv_write: v_first must be [n, kv_heads * dv]")
+        if v_first_mode == 2:
+            _check(v_mix is not None and v_mix.numel() == 1 and v_mix.dtype == v.dtype, "kv_write: v_mix is one element")
+    _i32(positions, "kv_write positions", n)
+    half = table_positions = 0
+    if cos is not None:
+        _check(cos.shape == sin.shape and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous()
+               and cos.dtype == sin.dtype == torch.float32, "kv_write: cos/sin tables")
+        table_positions, half = cos.shape
+    has_k = k is not None
+    lib.core().call("hfee_kv_write", _ptr(q), ldq, num_heads, q_dim, q_rot_offset, _ptr(k), ldk, k_rot_offset,
+                    _ptr(v), ldv, _ptr(v_first if has_k else None), v_first_mode if has_k else 0,
+                    _ptr(v_mix if has_k else None), _dt(some), _ptr(positions),
+                    _ptr(token_segment if has_k else None), _ptr(block_tables if has_k else None),
+                    block_tables.stride(0) if has_k else 0, _ptr(cos), _ptr(sin), half, table_positions,
+                    int(max_position), _ptr(cache_layer if has_k else None), kv_heads, dk, dv, page_size, n, _stream())
+
+
+def attention_kv_plain(out, q, cache_layer, positions, token_segment, block_tables, num_heads: int, kv_heads: int,
+                       dk: int, dv: int, page_size: int, scale: float, sinks=None):
+    """One wave per (token, head), any sizes, both dtypes: token t of head h reads the keys
+    0..pos of its sequence; `sinks` (float32 [num_heads] or None) joins the softmax's denominator."""
+    _gpu(out, q, cache_layer, positions, token_segment, block_tables, sinks)
+    n, w, ldq = _rows2d(q, "attention_kv q")
+    no, wo, ldo = _rows2d(out, "attention_kv out")
+    _check(no == n and w == num_heads * dk and wo == num_heads * dv, "attention_kv: q/out shape")
+    _check(q.dtype == out.dtype == cache_layer.dtype, "attention_kv: dtype mismatch")
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv")
+    _i32(positions, "attention_kv positions", n)
+    _i32(token_segment, "attention_kv token_segment", n)
+    _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+           "attention_kv: block tables")
+    if sinks is not None:
+        _check(sinks.dtype == torch.float32 and sinks.is_contiguous() and sinks.numel() == num_heads,
+               "attention_kv: sinks must be float32 [num_heads]")
+    lib.core().call("hfee_attention_kv_plain", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _dt(q),
+                    _ptr(positions), _ptr(token_segment), _ptr(block_tables), block_tables.stride(0),
+                    num_heads, kv_heads, dk, dv, page_size, float(scale), _ptr(sinks), n, _stream())
+
+
+def attention_kv_sizes_fit(dk: int, dv: int) -> bool:
+    """Whether the matrix-core kernels take these key and value sizes (else: the plain kernel)."""
+    from . import build
+    return dk % 16 == 0 and dv % 16 == 0 and 16 <= dk <= build.ATTENTION_KV_MOST[0] and 16 <= dv <= build.ATTENTION_KV_MOST[1]
+
+
+def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: int) -> int:
+    return num_items * num_heads * splits * (4 + dv) if splits > 1 else 0
+
+
+def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_heads: int, kv_heads: int, dk: int,
+                      dv: int, page_size: int, scale: float, sinks=None, partial=None, splits: int = 1):
+    """Matrix-core attention, bfloat16.  items: int32 [count, 4] on the device (first row, rows,
+    first position, block-table row).  mode 0: an item is up to 16 consecutive tokens of a portion;
+    mode 1: an item is a single token (rows = 1), whose keys may be split over `splits` waves that
+    leave partial results in `partial` (float32, `attention_kv_partial_words`) for a joining kernel."""
+    _gpu(out, q, cache_layer, items, block_tables, sinks, partial)
+    n, w, ldq = _rows2d(q, "attention_kv q")
+    no, wo, ldo = _rows2d(out, "attention_kv out")
+    _check(no == n and w == num_heads * dk and wo == num_heads * dv, "attention_kv: q/out shape")
+    _check(q.dtype == out.dtype == cache_layer.dtype == torch.bfloat16, "attention_kv: bfloat16 tensors expected")
+    _kv_cache(cache_layer, kv_heads, dk, dv, page_size, "attention_kv")
+    _check(items.dtype == torch.int32 and items.dim() == 2 and items.shape[1] == 4 and items.is_contiguous(),
+           "attention_kv: items must be [count, 4] int32")
+    _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+           "attention_kv: block tables")
+    if sinks is not None:
+        _check(sinks.dtype == torch.float32 and sinks.is_contiguous() and sinks.numel() == num_heads,
+               "attention_kv: sinks must be float32 [num_heads]")
+    if partial is not None:
+        _check(partial.dtype == torch.float32 and partial.is_contiguous(), "attention_kv: float32 partial buffer expected")
+    lib.attention_kv_bf16(dk, dv).call(
+        "hfee_attention_kv_bf16", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(items), items.shape[0], int(mode),
+        _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, page_size, float(scale), _ptr(sinks),
+        _ptr(partial), 0 if partial is None else partial.numel(), int(splits), _stream())
+
+
+def head_linear(out, x, weight, heads: int, n_in: int, n_out: int, tail: int = 0, x_head_stride: int | None = None,
+                out_head_stride: int | None = None):
+    """Per head: out[t, h, :n_out] = weight[h].T @ x[t, h, :n_in] (weight [heads, n_in, n_out]), then
+    x[t, h, n_in : n_in + tail] copied behind.  x and out are 2-D with contiguous rows; a head's
+    elements start every x_head_stride / out_head_stride (default: n_in + tail, n_out + tail)."""
+    _gpu(out, x, weight)
+    xs = n_in + tail if x_head_stride is None else x_head_stride
+    os_ = n_out + tail if out_head_stride is None else out_head_stride
+    n, wx, ldx = _rows2d(x, "head_linear x")
+    no, wo, ldo = _rows2d(out, "head_linear out")
+    _check(no == n and wx >= (heads - 1) * xs + n_in + tail and wo >= (heads - 1) * os_ + n_out + tail,
+           "head_linear: rows too short for the heads")
+    _check(weight.is_contiguous() and tuple(weight.shape) == (heads, n_in, n_out), "head_linear: weight [heads, n_in, n_out]")
+    _check(x.dtype == out.dtype == weight.dtype, "head_linear: dtype mismatch")
+    lib.core().call("hfee_head_linear", _ptr(out), ldo, os_, _ptr(x), ldx, xs, _ptr(weight), _dt(x), heads, n_in, n_out,
+                    tail, n, _stream())
+
+
+# ----------------------------------------------- blocks that norm a sub-layer's output; biases
+
+ROW_ACTIVATIONS = {"none": 0, "relu2": 1, "relu": 2, "gelu_tanh": 3, "silu": 4}
+
+
+def norm_add(x, y, weight, eps: float, bias=None, next_out=None, next_weight=None, next_eps: float = 0.0):
+    """x (float32, the residual stream) += norm(y + bias) * weight, norm(z) = z / sqrt(mean(z^2) + eps);
+    with next_out also next_out = norm(x_new) * next_weight (eps next_eps), the input of the sub-layer
+    that follows.  y: [n, d] float32 or bfloat16, contiguous; both weights of one dtype."""
+    _gpu(x, y, weight, bias, next_out, next_weight)
+    n, d, _ = _rows2d(x, "norm_add x")
+    _check(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and tuple(y.shape) == (n, d),
+           "norm_add: contiguous x (float32) and y of one shape")
+    _check(weight.numel() == d and weight.is_contiguous(), "norm_add: weight width")
+    if bias is not None:
+        _check(bias.numel() == d and bias.is_contiguous(), "norm_add: bias width")
+    if next_out is not None:
+        _check(next_weight is not None and next_weight.numel() == d and next_weight.is_contiguous()
+               and next_weight.dtype == weight.dtype, "norm_add: the following norm's weight")
+        _check(next_out.is_contiguous() and tuple(next_out.shape) == (n, d), "norm_add: next_out shape")
+    lib.core().call("hfee_norm_add", _ptr(x), _ptr(y), _dt(y), _ptr(bias), 0 if bias is None else _dt(bias),
+                    _ptr(weight), _dt(weight), 0.0, float(eps), _ptr(next_out), 0 if next_out is None else _dt(next_out),
+                    _ptr(next_weight), float(next_eps), n, d, _stream())
+
+
+def bias_act(out, x, bias, activation: str = "none"):
+    """out = activation(x + bias), row by row; "relu2" is the square of relu."""
+    _gpu(out, x, bias)
+    _check(activation in ROW_ACTIVATIONS, f"bias_act: the activations are {sorted(ROW_ACTIVATIONS)}, not {activation!r}")
+    n, w, ldi = _rows2d(x, "bias_act x")
+    no, wo, ldo = _rows2d(out, "bias_act out")
+    _check(no == n and wo == w and out.dtype == x.dtype, "bias_act: shapes and dtypes of x and out")
+    if bias is not None:
+        _check(bias.numel() == w and bias.is_contiguous() and bias.dtype == x.dtype, "bias_act: bias")
+    lib.core().call("hfee_bias_act", _ptr(out), ldo, _ptr(x), ldi, _ptr(bias), _dt(x), n, w, ROW_ACTIVATIONS[activation],
+                    _stream())
+
+
+def rmsnorm_cols(out, x, weight, eps: float):
+    """out[r] = x[r] / sqrt(mean(x[r]^2) + eps) * weight over the columns of x, a 2-D view in the
+    engine's dtype with contiguous rows (a block of columns of a wider buffer); out may be x."""
+    _gpu(out, x, weight)
+    n, w, ldx = _rows2d(x, "rmsnorm_cols x")
+    no, wo, ldo = _rows2d(out, "rmsnorm_cols out")
+    _check(no == n and wo == w and out.dtype == x.dtype, "rmsnorm_cols: shapes and dtypes of x and out")
+    _check(weight.numel() == w and weight.is_contiguous(), "rmsnorm_cols: weight width")
+    lib.core().call("hfee_rmsnorm_cols", _ptr(out), ldo, _ptr(x), ldx, _dt(x), _ptr(weight), _dt(weight), 0.0, float(eps),
+                    n, w, _stream())

@@ -2,12 +2,19 @@
 
 "prenorm" is the reference's block (/root/reference/internal/llm/forward.go:79-115):
 x += mixer(norm(x)); x += feed_forward(norm(x)).
+
+"sandwich" norms a sub-layer's output as well before it adds it:
+x += norm_b(mixer(norm_a(x))); x += norm_d(feed_forward(norm_c(x))), with four norms of their own
+weights, and a layer may have no feed-forward.  The sub-layers write float32 rows
+(`forward_into`); one launch norms them, adds them to the stream and makes the norm of the new
+stream for whatever follows (`ops.norm_add`), across layers too.
 """
 from __future__ import annotations
 
 import torch
 
 from ..config.specs import LayerSpec
+from ..kernels import ops
 from .base import LazyNorm, Part, lookup, register_block
 
 
@@ -67,3 +74,87 @@ class PreNormBlock(Part):
             part.forward_add(ctx, x, h, *args, then=then)
         else:
             part.forward_add(ctx, x, h, *args)
+
+
+@register_block("sandwich")
+class SandwichBlock(Part):
+    """Tensor names by role: mixer_norm, mixer_post_norm, feed_forward_norm, feed_forward_post_norm
+    (the whole name behind the layer's prefix), mixer and feed_forward (prefixes)."""
+
+    def __init__(self, spec: LayerSpec, dtype: torch.dtype):
+        self.spec, self.dtype, self.hidden = spec, dtype, spec.hidden
+
+        def norm(norm_spec, role):
+            return lookup("norm", norm_spec.kind)(norm_spec, spec.name_of(role, role + ".weight"))
+        self.mixer_norm = norm(spec.mixer_norm, "mixer_norm")
+        self.mixer_post_norm = norm(spec.mixer_norm, "mixer_post_norm")
+        self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, spec.name_of("mixer", "mixer."), dtype)
+        self.feed_forward = self.feed_forward_norm = self.feed_forward_post_norm = None
+        if spec.feed_forward is not None:
+            self.feed_forward_norm = norm(spec.feed_forward_norm, "feed_forward_norm")
+            self.feed_forward_post_norm = norm(spec.feed_forward_norm, "feed_forward_post_norm")
+            self.feed_forward = lookup("feed_forward", spec.feed_forward.kind)(
+                spec.feed_forward, spec.name_of("feed_forward", "feed_forward."), dtype)
+        for n in (self.mixer_post_norm, self.feed_forward_post_norm):
+            if n is not None and getattr(n, "fused_form", None) is None:
+                raise ValueError("a sandwich block norms its sub-layers' outputs with y / sqrt(mean(y^2) + eps) * w")
+
+    def _own(self):
+        return [p for p in (self.mixer_norm, self.mixer, self.mixer_post_norm, self.feed_forward_norm, self.feed_forward,
+                            self.feed_forward_post_norm) if p is not None]
+
+    def parts(self):
+        return [q for p in self._own() for q in p.parts()]
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def key_layout(self):
+        return getattr(self.mixer, "key_layout", lambda: None)()
+
+    def tensor_specs(self):
+        return [s for p in self._own() for s in p.tensor_specs()]
+
+    def bind(self, tensors):
+        for p in self._own():
+            p.bind(tensors)
+
+    chains_norms = True
+
+    def begin(self, ctx, x):
+        return LazyNorm(ctx, self.mixer_norm, x)
+
+    @staticmethod
+    def _rows_of(part, ctx, h, width, *args):
+        """The sub-layer's output as float32 rows (not yet added anywhere)."""
+        y = ctx.rows("block.sublayer_rows", width, torch.float32)
+        if hasattr(part, "forward_into"):
+            part.forward_into(ctx, y, h if part.takes_lazy_norm else h.tensor(), *args)
+        else:           # a part that only knows how to add: into rows of zeros
+            y.zero_()
+            part.forward_add(ctx, y, h if part.takes_lazy_norm else h.tensor(), *args)
+        return y
+
+    @staticmethod
+    def _add_normed(ctx, x, y, post_norm, bias, following):
+        """x += post_norm(y + bias), and the norm that follows in the same launch where it is of the
+        same form and nobody has made it yet."""
+        weight, eps = post_norm.fused_form()
+        nxt = following.fusable() if following is not None else None
+        if nxt is not None and following._tensor is None and following.pending is None and nxt[0].dtype == weight.dtype:
+            out = ctx.rows("block.normed", x.shape[1])
+            ops.norm_add(x, y, weight, eps, bias=bias, next_out=out, next_weight=nxt[0], next_eps=nxt[1])
+            following._tensor = out
+        else:
+            ops.norm_add(x, y, weight, eps, bias=bias)
+
+    def forward(self, ctx, x, entry, h_in=None, h_next=None):
+        h = h_in if h_in is not None else self.begin(ctx, x)
+        y = self._rows_of(self.mixer, ctx, h, self.hidden, entry.cache, entry.writes_cache)
+        if self.feed_forward is None:
+            self._add_normed(ctx, x, y, self.mixer_post_norm, getattr(self.mixer, "output_bias", None), h_next)
+            return
+        h2 = LazyNorm(ctx, self.feed_forward_norm, x)
+        self._add_normed(ctx, x, y, self.mixer_post_norm, getattr(self.mixer, "output_bias", None), h2)
+        y = self._rows_of(self.feed_forward, ctx, h2, self.hidden)
+        self._add_normed(ctx, x, y, self.feed_forward_post_norm, getattr(self.feed_forward, "output_bias", None), h_next)

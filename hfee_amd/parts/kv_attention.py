@@ -1,0 +1,277 @@
+"""Two mixers over one family of attention kernels, whose keys and values have sizes of their own.
+
+"kv_attention": grouped attention.  H query heads over G key/value heads (query head h reads
+key/value head h // (H/G)), key size Dk, value size Dv; q and k are rotated in the first
+`rotary_dim` dims of each head (the position part's tables carry the amplitude of a stretched
+rotation); score = q.k * scale over the keys up to the token's own position; the softmax may have a
+sink, one learned number a head that joins the denominator only (`sink`); the values may be blended
+with those that the first blending layer of the model computed for the same token (`value_blend`:
+"source" keeps its values of the step for the layers behind it, "mix" writes
+(1 - t) v + t v_source with its own learned t, and the blended values are what the cache holds).
+
+"latent_attention": queries and keys/values through low-rank latents.  c_q = norm(W_dq h),
+q = W_uq c_q, laid out head by head as [plain dims | rotated dims]; W_dkv h gives the latent c
+(normed) and one rotated key part that all heads share; per head k = [W_uk c | rotated part],
+v = W_uv c.  Only c and the rotated part are cached, and the attention runs in the absorbed form:
+since q_plain . (W_uk,h c) = (W_uk,h^T q_plain) . c, the query of head h becomes
+[W_uk,h^T q_plain | q_rotated] against the one cached row [c | rotated part] (one key/value head of
+size rank + rotated dims), the weighted sum is taken over the latents themselves (value size =
+rank), and W_uv,h is applied to the result.  Prompt portions and single tokens then run the same
+kernels, and a token's logits do not depend on how its prompt was cut.
+
+Both write float32 rows for a block that norms a sub-layer's output before it adds it to the
+residual stream (`forward_into`); `forward_add` is there for the other blocks.
+
+In bfloat16 with sizes that are multiples of 16 the matrix-core kernels run (rows of a prompt
+portion in tiles of 16, single tokens with the heads of a key/value head as the tile's rows and
+the keys split over waves); any other size, and float32, goes through the plain kernel.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..config.specs import CacheNeed, MixerSpec
+from ..kernels import ops
+from ..weights.spec import TensorSpec
+from .base import LazyNorm, Mixer, lookup, register_mixer
+
+_ROWS = 16             # query rows of a matrix-core tile
+_KEY_TILE = 32         # keys of a step of the matrix-core kernels
+_WAVES_WANTED = 2048   # single tokens split their keys until about this many waves run
+_MOST_SPLITS = 64
+_LAYOUT = "keys by slot, then values by dimension"
+
+
+def plan_items(plan) -> None:
+    """The step's work for the matrix-core kernels, once a step whichever layers ask: portions in
+    tiles of 16 rows, single tokens one by one (first row, rows, first position, block-table row)."""
+    if "attention_kv.portions" in plan.arrays:
+        return
+    portions, singles = [], []
+    for s, seg in enumerate(plan.segments):
+        if seg.length == 1:
+            singles.append((seg.row0, 1, seg.start, s))
+        else:
+            for off in range(0, seg.length, _ROWS):
+                portions.append((seg.row0 + off, min(_ROWS, seg.length - off), seg.start + off, s))
+    plan.add("attention_kv.portions", np.asarray(portions, dtype=np.int32).reshape(-1, 4))
+    plan.add("attention_kv.singles", np.asarray(singles, dtype=np.int32).reshape(-1, 4))
+    plan.host["attention_kv.single_max_position"] = max([p for _, _, p, _ in singles], default=0)
+
+
+def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks, matrix: bool) -> None:
+    if not matrix:
+        ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
+                               ctx.page_size, scale, sinks)
+        return
+    portions, singles = ctx.extra["attention_kv.portions"], ctx.extra["attention_kv.singles"]
+    if portions.shape[0]:
+        ops.attention_kv_bf16(out, q, cache, portions, 0, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks)
+    count = singles.shape[0]
+    if count:
+        # under a captured graph the split count is fixed for the whole width of the block table
+        span = ctx.host.get("graph.max_context", ctx.host["attention_kv.single_max_position"] + 1)
+        tiles = -(-span // _KEY_TILE)
+        units = kv_heads * -(-(num_heads // kv_heads) // _ROWS)
+        splits = max(1, min(tiles // 4, _WAVES_WANTED // (count * units), _MOST_SPLITS))
+        partial = None
+        if splits > 1:
+            partial = ctx.workspace.flat("attention_kv.partial", ops.attention_kv_partial_words(count, num_heads, dv, splits),
+                                         torch.float32)
+        ops.attention_kv_bf16(out, q, cache, singles, 1, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks,
+                              partial=partial, splits=splits)
+
+
+class _KvMixer(Mixer):
+    graph_safe = True
+
+    def _names(self, spec, defaults):
+        given = dict(spec.get("names") or ())
+        return {role: self.prefix + given.get(role, default) for role, default in defaults.items()}
+
+    def _matrix(self, dk, dv, q_width, out_width) -> bool:
+        return (self.dtype == torch.bfloat16 and ops.attention_kv_sizes_fit(dk, dv) and q_width % 8 == 0
+                and out_width % 4 == 0)
+
+    def prepare(self, info):
+        if self.position is not None:
+            self.position.prepare(info.num_positions, info.device)
+
+    def plan(self, plan):
+        if self.matrix:
+            plan_items(plan)
+
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
+        self.forward_into(ctx, y, h, cache_layer, writes_cache)
+        ops.residual_add(x, y)
+
+    def _tables(self, ctx, cache_layer):
+        return ctx.block_tables[ctx.storage.group_of(cache_layer)]
+
+
+@register_mixer("kv_attention")
+class KvAttention(_KvMixer):
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.num_heads = spec.get("num_heads")
+        self.kv_heads = spec.get("num_kv_heads", self.num_heads)
+        self.dk = spec.get("key_dim")
+        self.dv = spec.get("value_dim", self.dk)
+        self.scale = float(spec.get("scale", self.dk ** -0.5))
+        self.has_sink = bool(spec.get("sink", False))
+        self.blend = spec.get("value_blend")              # None | "source" | "mix"
+        if self.blend not in (None, "source", "mix"):
+            raise ValueError(f"value_blend is None, 'source' or 'mix', not {self.blend!r}")
+        if self.num_heads % self.kv_heads:
+            raise ValueError(f"{self.num_heads} heads are not a multiple of {self.kv_heads} kv heads")
+        self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
+        if self.position is not None and self.position.pairing != 0:
+            raise ValueError("kv_attention rotates pairs (i, i + half)")
+        self.names = self._names(spec, dict(q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", o="o_proj.weight",
+                                            sink="sinks", value_blend="value_blend"))
+        self.q_width, self.k_width, self.v_width = self.num_heads * self.dk, self.kv_heads * self.dk, self.kv_heads * self.dv
+        self.out_width = self.num_heads * self.dv
+        self.matrix = self._matrix(self.dk, self.dv, self.q_width + self.k_width + self.v_width, self.out_width)
+
+    def tensor_specs(self):
+        n = self.names
+        specs = [TensorSpec(n["q"], (self.q_width, self.hidden)), TensorSpec(n["k"], (self.k_width, self.hidden)),
+                 TensorSpec(n["v"], (self.v_width, self.hidden)), TensorSpec(n["o"], (self.hidden, self.out_width))]
+        if self.has_sink:
+            specs.append(TensorSpec(n["sink"], (self.num_heads,), role="vector"))
+        # (a layer that blends nothing may still carry the number in its checkpoint)
+        specs.append(TensorSpec(n["value_blend"], (), role="vector", optional=self.blend != "mix"))
+        return specs
+
+    def bind(self, tensors):
+        n = self.names
+        self.w_qkv = torch.cat([tensors.pop(n["q"]), tensors.pop(n["k"]), tensors.pop(n["v"])], dim=0).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.sinks = tensors.pop(n["sink"]).to(torch.float32).contiguous() if self.has_sink else None
+        t = tensors.pop(n["value_blend"], None)
+        self.blend_weight = t.reshape(1).to(self.dtype).contiguous() if (t is not None and self.blend == "mix") else None
+
+    def cache_spec(self):
+        return CacheNeed("full", (self.kv_heads, self.dk + self.dv), 0, layout=_LAYOUT)
+
+    def key_layout(self):
+        pos = self.position
+        return (self.kv_heads, self.dk, self.dv, None if pos is None else pos.signature())
+
+    def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
+        n = ctx.n
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        H, G, dk, dv = self.num_heads, self.kv_heads, self.dk, self.dv
+        cache = ctx.storage.layer(cache_layer, (G, ctx.page_size * (dk + dv)))
+        tables = self._tables(ctx, cache_layer)
+        pos = self.position
+        cos, sin = (pos.cos, pos.sin) if pos else (None, None)
+        qkv = ctx.rows("kv_attention.qkv", self.q_width + self.k_width + self.v_width)
+        q = qkv[:, :self.q_width]
+        if writes_cache:
+            ops.linear(qkv, hn, self.w_qkv, **ctx.workspace.split_scratch(n, self.w_qkv))
+            k = qkv[:, self.q_width:self.q_width + self.k_width]
+            v = qkv[:, self.q_width + self.k_width:]
+        else:       # this run of the layer reads keys and values that another run wrote
+            ops.linear(q, hn, self.w_qkv[:self.q_width])
+            k = v = None
+        first = None
+        if self.blend is not None and writes_cache:       # the source's values of this step's tokens
+            first = ctx.workspace.rows("kv_attention.blend_source", n, self.v_width, self.dtype)
+        ops.kv_write(q, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, cache, H, G, dk, dk, dv, ctx.page_size,
+                     ctx.max_position, v_first=first, v_first_mode={None: 0, "source": 1, "mix": 2}[self.blend],
+                     v_mix=self.blend_weight)
+        att = ctx.rows("kv_attention.out", self.out_width)
+        attend(ctx, att, q, cache, tables, H, G, dk, dv, self.scale, self.sinks, self.matrix)
+        ops.linear(out, att, self.w_o, **ctx.workspace.split_scratch(n, self.w_o))
+
+
+@register_mixer("latent_attention")
+class LatentAttention(_KvMixer):
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.num_heads = spec.get("num_heads")
+        self.plain = spec.get("plain_dim")
+        self.rotated = spec.get("rotated_dim")
+        self.dv = spec.get("value_dim", self.plain)
+        self.q_rank, self.kv_rank = spec.get("q_rank"), spec.get("kv_rank")
+        self.scale = float(spec.get("scale", (self.plain + self.rotated) ** -0.5))
+        self.eps = float(spec.get("norm_eps", 1e-6))
+        self.position = lookup("position", spec.position.kind)(spec.position) if spec.position else None
+        if self.position is not None and (self.position.pairing != 0 or self.position.rotary_dim != self.rotated):
+            raise ValueError("latent_attention rotates the whole rotated part, pairs (i, i + half)")
+        self.names = self._names(spec, dict(q_down="q_a_proj.weight", q_norm="q_a_norm.weight", q_up="q_b_proj.weight",
+                                            kv_down="kv_a_proj.weight", kv_norm="kv_a_norm.weight", k_up="k_b_proj.weight",
+                                            v_up="v_b_proj.weight", o="o_proj.weight"))
+        # the absorbed form: one key/value head, keys [latent | rotated part], values the latent
+        self.dk_abs, self.dv_abs = self.kv_rank + self.rotated, self.kv_rank
+        self.down_width = self.q_rank + self.kv_rank + self.rotated
+        self.matrix = (self._matrix(self.dk_abs, self.dv_abs, self.num_heads * self.dk_abs, self.num_heads * self.dv_abs)
+                       and self.down_width % 8 == 0 and self.q_rank % 8 == 0)
+
+    def tensor_specs(self):
+        n, H = self.names, self.num_heads
+        return [TensorSpec(n["q_down"], (self.q_rank, self.hidden)),
+                TensorSpec(n["q_norm"], (self.q_rank,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["q_up"], (H * (self.plain + self.rotated), self.q_rank)),
+                TensorSpec(n["kv_down"], (self.kv_rank + self.rotated, self.hidden)),
+                TensorSpec(n["kv_norm"], (self.kv_rank,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["k_up"], (H * self.plain, self.kv_rank)),
+                TensorSpec(n["v_up"], (H * self.dv, self.kv_rank)),
+                TensorSpec(n["o"], (self.hidden, H * self.dv))]
+
+    def bind(self, tensors):
+        n, H = self.names, self.num_heads
+        self.w_down = torch.cat([tensors.pop(n["q_down"]), tensors.pop(n["kv_down"])], dim=0).contiguous()
+        self.q_norm = tensors.pop(n["q_norm"]).to(torch.float32).contiguous()
+        self.kv_norm = tensors.pop(n["kv_norm"]).to(torch.float32).contiguous()
+        self.w_q_up = tensors.pop(n["q_up"]).contiguous()
+        # per head, as [inputs][outputs]: W_uk,h^T maps the plain query dims onto the latent, W_uv,h the
+        # weighted latent onto the head's values
+        self.w_k_absorb = tensors.pop(n["k_up"]).view(H, self.plain, self.kv_rank).contiguous()
+        self.w_v_expand = tensors.pop(n["v_up"]).view(H, self.dv, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+
+    def cache_spec(self):
+        return CacheNeed("full", (1, self.dk_abs + self.dv_abs), 0, layout=_LAYOUT)
+
+    def key_layout(self):
+        pos = self.position
+        return (1, self.dk_abs, self.dv_abs, None if pos is None else pos.signature())
+
+    def forward_into(self, ctx, out, h, cache_layer: int, writes_cache: bool):
+        n, H = ctx.n, self.num_heads
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        R, Dr, Dn = self.kv_rank, self.rotated, self.plain
+        dk, dv = self.dk_abs, self.dv_abs
+        cache = ctx.storage.layer(cache_layer, (1, ctx.page_size * (dk + dv)))
+        tables = self._tables(ctx, cache_layer)
+        pos = self.position
+        cos, sin = (pos.cos, pos.sin) if pos else (None, None)
+        down = ctx.rows("latent.down", self.down_width)
+        if writes_cache:
+            ops.linear(down, hn, self.w_down, **ctx.workspace.split_scratch(n, self.w_down))
+        else:
+            ops.linear(down[:, :self.q_rank], hn, self.w_down[:self.q_rank])
+        cq = ctx.rows("latent.q_latent", self.q_rank)
+        ops.rmsnorm_cols(cq, down[:, :self.q_rank], self.q_norm, self.eps)
+        q = ctx.rows("latent.q", H * (Dn + Dr))
+        ops.linear(q, cq, self.w_q_up, **ctx.workspace.split_scratch(n, self.w_q_up))
+        qa = ctx.rows("latent.q_absorbed", H * dk)
+        ops.head_linear(qa, q, self.w_k_absorb, H, Dn, R, tail=Dr)
+        k = v = None
+        if writes_cache:
+            c = down[:, self.q_rank:self.q_rank + R]
+            ops.rmsnorm_cols(c, c, self.kv_norm, self.eps)
+            k, v = down[:, self.q_rank:], c
+        ops.kv_write(qa, k, v, ctx.positions, ctx.token_segment, tables, cos, sin, cache, H, 1, dk, dk, dv, ctx.page_size,
+                     ctx.max_position, q_rot_offset=R, k_rot_offset=R)
+        att = ctx.rows("latent.mixed", H * dv)
+        attend(ctx, att, qa, cache, tables, H, 1, dk, dv, self.scale, None, self.matrix)
+        heads_out = ctx.rows("latent.values", H * self.dv)
+        ops.head_linear(heads_out, att, self.w_v_expand, H, R, self.dv)
+        ops.linear(out, heads_out, self.w_o, **ctx.workspace.split_scratch(n, self.w_o))

@@ -4,7 +4,12 @@ the residual stream; the reference's activation is the SiLU, and which one it is
 parameter of the part (`activation`: one of `ops.GATE_ACTIVATIONS`).  gate and up run as
 one product over a weight whose rows alternate gate_j, up_j, so that the gate is the
 product's epilogue (and a step of at most 64 tokens folds the norm in front of it into
-the same launch)."""
+the same launch).
+
+"dense_mlp" is the feed-forward without a gate: down(activation(up(h) + b_up)) + b_down, the
+activation one of `ops.ROW_ACTIVATIONS` ("relu2": the square of relu), the biases optional.  It
+writes float32 rows (`forward_into`) and leaves the last bias to whoever adds the rows to the
+residual stream (`output_bias`): a block that norms them first folds it into that launch."""
 from __future__ import annotations
 
 import torch
@@ -95,3 +100,52 @@ class GatedMLP(FeedForward):
             ops.linear_add_norm(x, act, self.w_down, after["out"], after["weight"], after["eps"], **cut)
         else:
             ops.linear(x, act, self.w_down, accumulate=True, **cut)
+
+
+@register_feed_forward("dense_mlp")
+class DenseMLP(FeedForward):
+    graph_safe = True
+
+    def __init__(self, spec: FeedForwardSpec, prefix: str, dtype: torch.dtype):
+        self.hidden = spec.get("hidden")
+        self.intermediate = spec.get("intermediate")
+        self.activation = spec.get("activation", "relu2")
+        self.has_bias = bool(spec.get("bias", False))
+        if self.activation not in ops.ROW_ACTIVATIONS:
+            raise ValueError(f"the dense feed-forward has the activations {sorted(ops.ROW_ACTIVATIONS)}, "
+                             f"not {self.activation!r}")
+        self.prefix, self.dtype = prefix, dtype
+        given = dict(spec.get("names") or ())
+        defaults = dict(up="up_proj.weight", up_bias="up_proj.bias", down="down_proj.weight", down_bias="down_proj.bias")
+        self.names = {role: prefix + given.get(role, default) for role, default in defaults.items()}
+        self.output_bias = None          # float32; added by whoever takes the rows of forward_into
+
+    def tensor_specs(self):
+        n = self.names
+        specs = [TensorSpec(n["up"], (self.intermediate, self.hidden)), TensorSpec(n["down"], (self.hidden, self.intermediate))]
+        if self.has_bias:
+            specs += [TensorSpec(n["up_bias"], (self.intermediate,), role="vector"),
+                      TensorSpec(n["down_bias"], (self.hidden,), role="vector")]
+        return specs
+
+    def bind(self, tensors):
+        n = self.names
+        self.w_up, self.w_down = tensors.pop(n["up"]).contiguous(), tensors.pop(n["down"]).contiguous()
+        self.up_bias = tensors.pop(n["up_bias"]).to(self.dtype).contiguous() if self.has_bias else None
+        self.output_bias = tensors.pop(n["down_bias"]).to(torch.float32).contiguous() if self.has_bias else None
+
+    def forward_into(self, ctx, out, h):
+        """out (float32 [n, hidden]) = down(activation(up(h) + b_up)); `output_bias` is not added."""
+        n = ctx.n
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        act = ctx.rows("dense_mlp.act", self.intermediate)
+        ops.linear(act, hn, self.w_up, **ctx.workspace.split_scratch(n, self.w_up))
+        ops.bias_act(act, act, self.up_bias, self.activation)
+        ops.linear(out, act, self.w_down, **ctx.workspace.split_scratch(n, self.w_down))
+
+    def forward_add(self, ctx, x, h):
+        y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
+        self.forward_into(ctx, y, h)
+        if self.output_bias is not None:
+            ops.bias_act(y, y, self.output_bias, "none")
+        ops.residual_add(x, y)

@@ -1,7 +1,11 @@
 """RMSNorm (/root/reference/internal/ggml/ops.go:124-134): y = x / sqrt(mean(x^2) + eps) * w,
-the sum in float32, x the float32 residual stream, y in the engine's dtype; and "none" for a
+the sum in float32, x the float32 residual stream, y in the engine's dtype (with the parameter
+`weight_offset` the stored weight lies around zero and the norm multiplies by offset + w: the sum
+is made once, in float32, when the weight is bound); and "none" for a
 place where a model has no norm (the rows as they are, in the engine's dtype)."""
 from __future__ import annotations
+
+import torch
 
 from ..config.specs import NormSpec
 from ..kernels import ops
@@ -15,13 +19,17 @@ class RMSNorm(Norm):
 
     def __init__(self, spec: NormSpec, name: str):
         self.width, self.eps, self.name = spec.width, spec.eps, name
+        self.offset = float(dict(spec.params).get("weight_offset", 0.0))
         self.weight = None
 
     def tensor_specs(self):
-        return [TensorSpec(self.name, (self.width,), role="vector", init=("one_plus_normal",))]
+        return [TensorSpec(self.name, (self.width,), role="vector",
+                           init=("normal",) if self.offset else ("one_plus_normal",))]
 
     def bind(self, tensors):
         self.weight = tensors[self.name]
+        if self.offset:
+            self.weight = (self.weight.to(torch.float32) + self.offset).contiguous()
 
     def fused_form(self):
         return self.weight, self.eps

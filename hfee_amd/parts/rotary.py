@@ -11,6 +11,13 @@ The reference takes sin and cos of the float64 angle position * inv_freq at ever
 use (/root/reference/internal/llm/forward.go:186).  Here a table [positions, dim/2]
 of cos and sin is made once from those float64 angles and rounded to float32, so
 large positions lose nothing to a float32 angle.
+
+A second stretching rule, "yarn": (kind, factor, original context, fast, slow).  With
+turn(t) = dim * ln(original / (2 pi t)) / (2 ln theta), the dimension whose wave makes t turns over
+the original context, the dimensions up to lo = max(floor(turn(fast)), 0) keep their frequency,
+those from hi = min(ceil(turn(slow)), dim - 1) on are divided by `factor`, and between them the
+two are blended linearly in the dimension's index; cos and sin are both scaled by
+0.1 ln(factor) + 1 (`rope_amplitude`), which the tables carry.
 """
 from __future__ import annotations
 
@@ -30,6 +37,15 @@ def rope_frequencies(rotary_dim: int, theta: float, scaling=None) -> np.ndarray:
     inv = np.array([1.0 / math.pow(theta, (2 * i) / rotary_dim) for i in range(half)], dtype=np.float64)
     if scaling is None:
         return inv
+    if scaling[0] == "yarn":
+        _, factor, original, fast, slow = scaling
+
+        def turn(t):
+            return rotary_dim * math.log(original / (2 * math.pi * t)) / (2 * math.log(theta))
+        lo = max(math.floor(turn(fast)), 0)
+        hi = min(math.ceil(turn(slow)), rotary_dim - 1)
+        ramp = np.clip((np.arange(half, dtype=np.float64) - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return inv / factor * ramp + inv * (1.0 - ramp)
     kind, factor, low, high, original = scaling
     if kind != "llama3":
         raise ValueError(f"unknown rope scaling {kind!r}")
@@ -46,6 +62,13 @@ def rope_frequencies(rotary_dim: int, theta: float, scaling=None) -> np.ndarray:
     return out
 
 
+def rope_amplitude(scaling=None) -> float:
+    """What cos and sin are multiplied by: 1, but 0.1 ln(factor) + 1 under the "yarn" rule."""
+    if scaling is not None and scaling[0] == "yarn":
+        return 0.1 * math.log(float(scaling[1])) + 1.0
+    return 1.0
+
+
 @register_position("rope")
 class Rotary(Part):
     def __init__(self, spec: PositionSpec):
@@ -60,6 +83,7 @@ class Rotary(Part):
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {self.head_dim}")
         self.pairing = PAIRINGS[pairing]
         self.inv_freq = rope_frequencies(self.rotary_dim, self.theta, self.scaling)
+        self.amplitude = rope_amplitude(self.scaling)
         self.cos = self.sin = None
 
     def signature(self):
@@ -70,5 +94,5 @@ class Rotary(Part):
         if self.cos is not None and self.cos.shape[0] >= num_positions and self.cos.device == torch.device(device):
             return
         angles = np.arange(num_positions, dtype=np.float64)[:, None] * self.inv_freq[None, :]
-        self.cos = torch.from_numpy(np.cos(angles).astype(np.float32)).to(device)
-        self.sin = torch.from_numpy(np.sin(angles).astype(np.float32)).to(device)
+        self.cos = torch.from_numpy((np.cos(angles) * self.amplitude).astype(np.float32)).to(device)
+        self.sin = torch.from_numpy((np.sin(angles) * self.amplitude).astype(np.float32)).to(device)
