@@ -1,0 +1,364 @@
+"""The Vofezen decoder on the GPU against the plain implementation: every new kernel alone, the
+whole model under four ways of cutting the same requests into steps (whole, bulk then single
+tokens, portions down to two tokens, mixed batches on a small page pool whose pages are used
+again), in 32-bit and in bfloat16, on configurations with sizes that the matrix-core kernels take
+and sizes that they do not; long decoding through graph replays; greedy generation through the
+entry point and its scheduler; the trace runner as a subprocess."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_vofezen as pv
+import trace_util as tu
+import vofezen_util as vu
+from conftest import ROOT
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"float32": 3e-5, "bfloat16": 5e-2}
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+LENGTHS = {"A": [5, 17, 64, 1, 100, 33, 129, 49, 2], "B": [40, 3, 100, 65, 2, 31], "C": [150, 70, 700, 41, 97]}
+
+
+def dev(a, dtype=None):
+    t = torch.as_tensor(np.asarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda().contiguous()
+
+
+def as_bf16(a):
+    """float64 numpy rounded to bfloat16 and back (what a bfloat16 tensor of it holds)."""
+    return torch.as_tensor(np.asarray(a, dtype=np.float32)).to(torch.bfloat16).double().numpy()
+
+
+# ------------------------------------------------------------------ kernels alone
+
+class PagedCase:
+    """Sequences with tokens already in a paged cache and new tokens in a step: pages in a
+    shuffled order, block tables, positions, as the engine would hand them to the kernels."""
+
+    def __init__(self, starts, lengths, kv_heads, dk, dv, dtype, page_size=16, seed=0):
+        from hfee_amd.kernels import ops
+        self.ops = ops
+        rng = np.random.default_rng(seed)
+        self.page_size, self.G, self.dk, self.dv, self.dtype = page_size, kv_heads, dk, dv, dtype
+        totals = [s + l for s, l in zip(starts, lengths)]
+        blocks = [-(-t // page_size) for t in totals]
+        pages = rng.permutation(sum(blocks) + 3)
+        self.tables = np.zeros((len(starts), max(blocks)), dtype=np.int32)
+        at = 0
+        for i, b in enumerate(blocks):
+            self.tables[i, :b] = pages[at:at + b]
+            at += b
+        # (stale numbers in every page, as a pool that has been used before holds them)
+        self.cache = dev(rng.standard_normal((len(pages), kv_heads, page_size * (dk + dv))) * 3, dtype)
+        self.starts, self.lengths, self.totals = starts, lengths, totals
+        self.d_tables = dev(self.tables)
+
+    def write(self, seq, first, k, v, q=None, cos=None, sin=None, **kw):
+        """Writes k, v (and rotates q) for positions first.. of sequence seq as one step."""
+        n = k.shape[0]
+        pos = dev(np.arange(first, first + n, dtype=np.int32))
+        seg = dev(np.full(n, seq, dtype=np.int32))
+        H = 0 if q is None else q.shape[1] // kw.pop("q_dim", self.dk)
+        q_dim = 0 if q is None else q.shape[1] // H
+        self.ops.kv_write(q, k, v, pos, seg, self.d_tables, cos, sin, self.cache, H, self.G, q_dim, self.dk, self.dv,
+                          self.page_size, first + n - 1, **kw)
+
+
+def softmax_rows(q, k, v, scale, positions, sink=None):
+    """q [n, H, dk] at `positions` of a sequence with keys k [T, G, dk], values v [T, G, dv]."""
+    n, H, _ = q.shape
+    G = k.shape[1]
+    out = np.zeros((n, H, v.shape[2]))
+    for i in range(n):
+        for h in range(H):
+            g = h // (H // G)
+            s = (k[:positions[i] + 1, g] @ q[i, h]) * scale
+            m = max(s.max(), sink[h]) if sink is not None else s.max()
+            e = np.exp(s - m)
+            den = e.sum() + (np.exp(sink[h] - m) if sink is not None else 0.0)
+            out[i, h] = (e / den) @ v[:positions[i] + 1, g]
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,G,dk,dv", [(4, 2, 32, 16), (20, 1, 16, 48), (3, 3, 24, 28), (6, 1, 128, 96), (5, 5, 64, 64)])
+def test_attention_kernels(dtype, H, G, dk, dv):
+    """Plain and matrix-core kernels, portions and single tokens (keys split and not), a sink, stale
+    numbers in the pages, one far key that outweighs hundreds, and a sink that outweighs all keys."""
+    from hfee_amd.kernels import ops
+    dt = DT[dtype]
+    rng = np.random.default_rng(H * 100 + dk)
+    starts, lengths = [0, 37, 600, 15], [45, 19, 1, 1]
+    case = PagedCase(starts, lengths, G, dk, dv, dt, seed=dk)
+    scale = 0.8 / dk ** 0.5
+    keys, values, queries = [], [], []
+    for s, (st, ln) in enumerate(zip(starts, lengths)):
+        T = st + ln
+        k, v = rng.standard_normal((T, G, dk)), rng.standard_normal((T, G, dv))
+        q = rng.standard_normal((ln, H, dk))
+        if s == 2:            # one key far back decides the last token of the long sequence
+            k[5] *= 5.0
+            mine = k[5, np.arange(H) // (H // G)]
+            q[-1] = 20.0 * mine / scale / (mine ** 2).sum(-1, keepdims=True)
+        if dtype == "bfloat16":
+            k, v, q = as_bf16(k), as_bf16(v), as_bf16(q)
+        keys.append(k), values.append(v), queries.append(q)
+        case.write(s, 0, dev(k.reshape(T, -1), dt), dev(v.reshape(T, -1), dt))
+    sink = rng.standard_normal(H) * 2
+    sink[0] = 30.0            # head 0: the sink takes nearly everything
+    n = sum(lengths)
+    q_all = dev(np.concatenate([q.reshape(q.shape[0], -1) for q in queries]), dt)
+    positions = np.concatenate([np.arange(st, st + ln) for st, ln in zip(starts, lengths)]).astype(np.int32)
+    segment = np.repeat(np.arange(len(starts)), lengths).astype(np.int32)
+    want = np.concatenate([softmax_rows(q, k, v, scale, np.arange(st, st + ln), sink)
+                           for q, k, v, st, ln in zip(queries, keys, values, starts, lengths)]).reshape(n, -1)
+    no_sink = np.concatenate([softmax_rows(q, k, v, scale, np.arange(st, st + ln))
+                              for q, k, v, st, ln in zip(queries, keys, values, starts, lengths)]).reshape(n, -1)
+    assert np.abs(want[:, :dv]).max() < 1e-3 * np.abs(no_sink[:, :dv]).max()      # the sink shows
+    far = softmax_rows(queries[2], keys[2], values[2], scale, [600])[0]
+    assert vu.rel(far[0], values[2][5, 0]) < 0.05                                       # and so does the far key
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    d_sink = dev(sink, torch.float32)
+    out = torch.zeros((n, H * dv), dtype=dt, device="cuda")
+    ops.attention_kv_plain(out, q_all, case.cache, dev(positions), dev(segment), case.d_tables, H, G, dk, dv, 16, scale, d_sink)
+    assert vu.rel(out.double().cpu(), want) < tol
+    out.zero_()
+    ops.attention_kv_plain(out, q_all, case.cache, dev(positions), dev(segment), case.d_tables, H, G, dk, dv, 16, scale, None)
+    assert vu.rel(out.double().cpu(), no_sink) < tol
+    if dtype == "float32" or not ops.attention_kv_sizes_fit(dk, dv):
+        return
+    items0, row = [], 0
+    for s, (st, ln) in enumerate(zip(starts, lengths)):
+        if ln > 1:
+            items0 += [(row + off, min(16, ln - off), st + off, s) for off in range(0, ln, 16)]
+        row += ln
+    items1 = [(64, 1, 600, 2), (65, 1, 15, 3)]
+    for sinks, ref in ((d_sink, want), (None, no_sink)):
+        for splits in (1, 3, 64):
+            out.zero_()
+            ops.attention_kv_bf16(out, q_all, case.cache, dev(np.asarray(items0, dtype=np.int32)), 0, case.d_tables, H, G, dk, dv,
+                                  16, scale, sinks)
+            partial = torch.full((ops.attention_kv_partial_words(2, H, dv, splits),), float("nan"), device="cuda") if splits > 1 else None
+            ops.attention_kv_bf16(out, q_all, case.cache, dev(np.asarray(items1, dtype=np.int32)), 1, case.d_tables, H, G, dk, dv,
+                                  16, scale, sinks, partial=partial, splits=splits)
+            assert vu.rel(out.double().cpu(), ref) < tol, (splits, sinks is None)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cache_write_rotates_and_blends(dtype):
+    from hfee_amd.kernels import ops
+    dt = DT[dtype]
+    rng = np.random.default_rng(2)
+    H, G, dk, dv, dims, off = 3, 2, 20, 12, 8, 6
+    n, first = 21, 27
+    case = PagedCase([first], [n], G, dk, dv, dt)
+    q, k, v = rng.standard_normal((n, H, dk)), rng.standard_normal((n, G, dk)), rng.standard_normal((n, G, dv))
+    v0 = rng.standard_normal((n, G, dv))
+    if dtype == "bfloat16":
+        q, k, v, v0 = as_bf16(q), as_bf16(k), as_bf16(v), as_bf16(v0)
+    freq, amp = pv.rotary_frequencies(dims, 100.0, {"factor": 2.0, "original": 16, "fast": 4.0, "slow": 1.0})
+    pos = np.arange(first, first + n)
+    angles = np.arange(64)[:, None] * freq[None]
+    cos, sin = dev(np.cos(angles) * amp, torch.float32), dev(np.sin(angles) * amp, torch.float32)
+
+    def rotated(u):
+        out = u.copy()
+        out[..., off:] = pv.rotate(u[..., off:], pos, freq, amp, dims)
+        return out
+    lam = 0.375
+    dq, dfirst = dev(q.reshape(n, -1), dt), dev(v0.reshape(n, -1), dt)
+    case.write(0, first, dev(k.reshape(n, -1), dt), dev(v.reshape(n, -1), dt), q=dq, cos=cos, sin=sin, q_rot_offset=off,
+               k_rot_offset=off, v_first=dfirst, v_first_mode=2, v_mix=dev([lam], dt))
+    tol = 1e-6 if dtype == "float32" else 1e-2
+    assert vu.rel(dq.double().cpu().reshape(n, H, dk), rotated(q)) < tol
+    cache = case.cache.double().cpu().numpy()
+    kw, vw = rotated(k), (1 - lam) * v + lam * v0
+    for i, p in enumerate(pos):
+        page, slot = case.tables[0, p // 16], p % 16
+        for g in range(G):
+            block = cache[page, g]
+            assert vu.rel(block[slot * dk:(slot + 1) * dk], kw[i, g]) < tol
+            assert vu.rel(block[16 * dk:].reshape(dv, 16)[:, slot], vw[i, g]) < tol
+    # mode 1 hands the values on as they are
+    case.write(0, first, dev(k.reshape(n, -1), dt), dev(v.reshape(n, -1), dt), v_first=dfirst, v_first_mode=1)
+    np.testing.assert_array_equal(dfirst.double().cpu().numpy(), dev(v.reshape(n, -1), dt).double().cpu().numpy())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_row_kernels(dtype):
+    from hfee_amd.kernels import ops
+    dt = DT[dtype]
+    rng = np.random.default_rng(4)
+    tol = 2e-6 if dtype == "float32" else 1e-2
+    n, d = 37, 58
+    x, y, b = rng.standard_normal((n, d)), rng.standard_normal((n, d)) * 3, rng.standard_normal(d)
+    w1, w2 = 1 + rng.standard_normal(d) * 0.3, 1 + rng.standard_normal(d) * 0.3
+    for y_dt in (torch.float32, dt):
+        yy = as_bf16(y) if y_dt == torch.bfloat16 else y
+        dx, nxt = dev(x, torch.float32), torch.zeros((n, d), dtype=dt, device="cuda")
+        ops.norm_add(dx, dev(yy, y_dt), dev(w1, torch.float32), 1e-5, bias=dev(b, torch.float32), next_out=nxt,
+                     next_weight=dev(w2, torch.float32), next_eps=1e-3)
+        want = x + pv.unit_rms(yy + b, 1e-5) * w1
+        assert vu.rel(dx.double().cpu(), want) < 2e-6
+        assert vu.rel(nxt.double().cpu(), pv.unit_rms(want, 1e-3) * w2) < tol
+        dx = dev(x, torch.float32)
+        ops.norm_add(dx, dev(yy, y_dt), dev(w1, torch.float32), 1e-5)
+        assert vu.rel(dx.double().cpu(), x + pv.unit_rms(yy, 1e-5) * w1) < 2e-6
+    z, zb = (as_bf16(a) if dtype == "bfloat16" else a for a in (y, b))
+    for act, f in (("relu2", lambda t: np.maximum(t, 0) ** 2), ("none", lambda t: t), ("relu", lambda t: np.maximum(t, 0)),
+                   ("gelu_tanh", lambda t: 0.5 * t * (1 + np.tanh(np.sqrt(2 / np.pi) * (t + 0.044715 * t ** 3)))),
+                   ("silu", lambda t: t / (1 + np.exp(-t)))):
+        out = torch.zeros((n, d), dtype=dt, device="cuda")
+        ops.bias_act(out, dev(z, dt), dev(zb, dt), act)
+        assert vu.rel(out.double().cpu(), f(z + zb)) < tol, act
+    wide = dev(z, dt)
+    cols = wide[:, 7:47]
+    w = 1 + rng.standard_normal(40) * 0.2
+    out = torch.zeros((n, 40), dtype=dt, device="cuda")
+    ops.rmsnorm_cols(out, cols, dev(w, torch.float32), 1e-5)
+    assert vu.rel(out.double().cpu(), pv.unit_rms(z[:, 7:47], 1e-5) * w) < tol
+    ops.rmsnorm_cols(cols, cols, dev(w, torch.float32), 1e-5)            # in place, the neighbours untouched
+    assert vu.rel(wide.double().cpu()[:, 7:47], pv.unit_rms(z[:, 7:47], 1e-5) * w) < tol
+    before = dev(z, dt).double().cpu().numpy()
+    np.testing.assert_array_equal(wide.double().cpu().numpy()[:, :7], before[:, :7])
+    np.testing.assert_array_equal(wide.double().cpu().numpy()[:, 47:], before[:, 47:])
+    # per-head products, with a tail carried along
+    heads, n_in, n_out, tail = 5, 12, 40, 6
+    xh, wh = rng.standard_normal((n, heads, n_in + tail)), rng.standard_normal((heads, n_in, n_out))
+    if dtype == "bfloat16":
+        xh, wh = as_bf16(xh), as_bf16(wh)
+    out = torch.zeros((n, heads * (n_out + tail)), dtype=dt, device="cuda")
+    ops.head_linear(out, dev(xh.reshape(n, -1), dt), dev(wh, dt), heads, n_in, n_out, tail=tail)
+    want = np.concatenate([np.einsum("thi,hio->tho", xh[..., :n_in], wh), xh[..., n_in:]], axis=-1)
+    assert vu.rel(out.double().cpu().reshape(n, heads, -1), want) < tol
+
+
+# ------------------------------------------------------------------ the whole model
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    base = tmp_path_factory.mktemp("vofezen")
+    return {(name, dtype): vu.make_folder(base / f"{name}_{dtype}", cj, seed=7 + ord(name), dtype=dtype)
+            for name, cj in vu.CONFIGS.items() for dtype in ("float32", "bfloat16")}
+
+
+@pytest.fixture(scope="module")
+def plain_rows(folders):
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            reqs = tu.make_requests(vu.CONFIGS[name]["vocab"], LENGTHS[name], seed=ord(name))
+            model = pv.PlainVofezen(folders[(name, dtype)])
+            rows = {}
+            for rid, toks in reqs.items():
+                logits = model.forward(toks)
+                rows.update({(rid, i): logits[i] for i in range(len(toks))})
+            cache[(name, dtype)] = (reqs, rows)
+        return cache[(name, dtype)]
+    return get
+
+
+def compare(got, want, tol, what):
+    assert set(got) == set(want), f"{what}: positions differ"
+    worst, where = 0.0, None
+    for key in want:
+        e = vu.rel(got[key], want[key])
+        if not e <= worst:
+            worst, where = e, key
+    assert worst < tol, f"{what}: worst relative error {worst:.3e} at {where}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_every_way_of_cutting_gives_the_plain_logits(folders, plain_rows, name, dtype):
+    from hfee_amd.trace_replay import Replayer
+    reqs, want = plain_rows(name, dtype)
+    longest = max(len(t) for t in reqs.values())
+    one = (longest + 63) // 64 * 64
+    for what, steps, room in (("whole", tu.whole(reqs), one), ("bulk then single tokens", tu.bulk_then_tail(reqs, 40), one),
+                              ("portions", tu.portions(reqs), one), ("mixed", *tu.mixed(reqs, seed=len(name)))):
+        rep = Replayer(folders[(name, dtype)], dtype, room, max_requests=4)
+        got = tu.run(rep, steps)
+        compare(got, want, TOL[dtype], f"{name} {dtype} {what}")
+        rep.engine.cache.check()
+        assert not rep.engine.cache.requests
+
+
+def test_cuts_agree_closely_in_32_bit(folders, plain_rows):
+    """Whole prompts against portions and single tokens: rounding apart, the same logits."""
+    from hfee_amd.trace_replay import Replayer
+    reqs, _ = plain_rows("A", "float32")
+    runs = []
+    for steps in (tu.whole(reqs), tu.portions(reqs, sizes=(2, 3, 16, 1, 15, 17, 2)), tu.bulk_then_tail(reqs, 20)):
+        runs.append(tu.run(Replayer(folders[("A", "float32")], "float32", 192, max_requests=4), steps))
+    for other in runs[1:]:
+        for key in runs[0]:
+            assert vu.rel(other[key], runs[0][key]) < 2e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(folders, dtype):
+    """300 single tokens after a short prompt: decode steps replayed from captured graphs, across
+    page borders, the split count of the single-token kernel growing with the context."""
+    from hfee_amd.trace_replay import Replayer
+    rng = np.random.default_rng(9)
+    toks = rng.integers(0, 300, size=330).tolist()
+    rep = Replayer(folders[("C", dtype)], dtype, 384, max_requests=4)
+    steps = [{"entries": [("a", toks[:30], [29])], "end": []}]
+    steps += [{"entries": [("a", toks[i:i + 1], [0])], "end": ["a"] if i == 329 else []} for i in range(30, 330)]
+    got = tu.run(rep, steps)
+    assert rep.engine.graph_replays > 250
+    want = pv.PlainVofezen(folders[("C", dtype)]).forward(toks)
+    compare(got, {("a", i): want[i] for i in range(29, 330)}, TOL[dtype], f"long decoding {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(folders, dtype):
+    from hfee_amd import LLM, SamplingParams
+    folder = folders[("A", dtype)]
+    plain = pv.PlainVofezen(folder)
+    llm = LLM(folder, dtype=dtype, num_ctx=128, num_parallel=3, max_batch_tokens=24)
+    g = np.random.default_rng(5)
+    prompts = [g.integers(0, 211, size=n).tolist() for n in (5, 40, 1, 17, 33)]
+    outs = llm.generate(prompts, SamplingParams.greedy(num_predict=8))
+    for p, o in zip(prompts, outs):
+        want = plain.greedy(p, 8)
+        if dtype == "float32":
+            assert o.token_ids == want
+        else:
+            logits = plain.forward(p + want)
+            margins = []
+            for i in range(8):
+                row = np.sort(logits[len(p) - 1 + i])
+                margins.append(float((row[-1] - row[-2]) / np.abs(row).max()))
+            tu.agree_until_a_near_tie(o.token_ids, want, margins, f"greedy {dtype}")
+
+
+def test_trace_runner_as_a_subprocess(folders, tmp_path):
+    folder = folders[("B", "float32")]
+    toks = list(range(1, 40))
+    lines = [{"step": 0, "entries": [{"id": "x", "tokens": toks[:21], "want": [0, 20]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": toks[21:22], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": toks[22:], "want": [16]}, {"id": "y", "tokens": toks[:2], "want": [1]}],
+              "end": ["x", "y"]}]
+    out = tmp_path / "out"
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", "float32",
+                        "--out", str(out), "--max-tokens", "128"], input="\n".join(json.dumps(l) for l in lines) + "\n",
+                       capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    want = pv.PlainVofezen(folder).forward(toks)
+    a = np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1)
+    c = np.fromfile(out / "2.f32", dtype="<f4").reshape(2, -1)
+    assert not (out / "1.f32").exists()
+    assert vu.rel(a[0], want[0]) < 3e-5 and vu.rel(a[1], want[20]) < 3e-5
+    assert vu.rel(c[0], want[38]) < 3e-5 and vu.rel(c[1], want[1]) < 3e-5
