@@ -49,6 +49,16 @@ SHAPES = {
 }
 SHAPE_NAMES = {"llama-3.1-8b": "Llama-3.1-8B", "llama-3.2-1b": "Llama-3.2-1B", "llama-2-13b": "Llama-2-13B",
                "llama-3.2-3b": "Llama-3.2-3B", "llama-2-7b": "Llama-2-7B", "llama-3.1-70b": "Llama-3.1-70B"}
+# Two layer sizes that resemble real models' layers.  A Vofezen layer of a size has the width,
+# heads and matrix parameters of the Llama layer beside it (two feed-forward matrices of 3/2 the
+# width of Llama's three); every fourth layer is latent attention with latents of 512 (keys) and
+# 1,536 or 768 (queries).
+VOFEZEN_SIZES = {
+    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=12288, llama_ff=8192, q_rank=768),
+    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, q_rank=1536),
+}
+
+
 CONTEXT = 8192
 PROMPT = 1024
 PREFILL = 2048
@@ -82,6 +92,14 @@ def parse(argv=None):
     ap.add_argument("--attention-alone", action="store_true",
                     help="only time the prefill attention kernel by itself: the last 2,048 rows of one sequence of "
                          "2,048, 8,192 and 32,768 tokens (heads and head size of --shape); prints its own line")
+    ap.add_argument("--vofezen", action="store_true",
+                    help="instead of the default run: the Vofezen design (sandwich blocks, attention with a sink and "
+                         "blended values, latent attention, dense feed-forward) at two layer sizes beside the Llama "
+                         "decoder at equal width, heads and parameters a layer; prints its own line")
+    ap.add_argument("--vofezen-size", choices=sorted(VOFEZEN_SIZES), default=None,
+                    help="with --vofezen: only this layer size")
+    ap.add_argument("--vofezen-design", choices=["both", "vofezen", "llama"], default="both",
+                    help="with --vofezen: only one of the two designs (for profiling)")
     ap.add_argument("--no-extra-points", action="store_true",
                     help="skip the other shapes and the longer context that the default run adds under `points`")
     return ap.parse_args(argv)
@@ -154,11 +172,121 @@ def attention_alone(shape: dict) -> dict:
     return out
 
 
+def vofezen_configs(size: dict, layers: int, vocab: int = 32000):
+    """(config.json keys of the Vofezen model, of the Llama model beside it)."""
+    d, H, G, hd = size["width"], size["heads"], size["kv_heads"], size["dim"]
+    rot = {"base": 500000.0, "dims": hd // 2, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": size["ff"]},
+           "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5, "v_mix": True, "rot": rot}}
+    lat = {"type": "latent_attention", "mlp": {"kind": "dense", "ff": size["ff"]},
+           "mixer": {"heads": H, "dim": hd, "rot_dim": 64, "vdim": hd, "q_rank": size["q_rank"], "kv_rank": 512,
+                     "scale": (hd + 64) ** -0.5, "rot": {"base": 500000.0, "dims": 64}}}
+    vof = {"architecture": "Vofezen", "vocab": vocab, "width": d, "norm": {"eps": 1e-5},
+           "layers": [lat if i % 4 == 2 else att for i in range(layers)]}
+    llama = dict(BASE_8B, architectures=["LlamaForCausalLM"], num_hidden_layers=layers, hidden_size=d,
+                 num_attention_heads=H, num_key_value_heads=G, head_dim=hd, intermediate_size=size["llama_ff"],
+                 vocab_size=vocab)
+    return vof, llama
+
+
+def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
+    """Prefill of 2,048 tokens and decode at `batch` requests of 1,024-token prompts for any
+    registered architecture: times, and the fractions of the HBM and matrix peaks by the bytes a
+    step must read (every matrix once, the cache of the live requests) and the flops of the
+    products and of the attention as the kernels run it."""
+    import torch
+
+    from hfee_amd.cache import bytes_per_token
+    from hfee_amd.config import config_from_dict
+    from hfee_amd.engine import Engine, Request, Scheduler, StepEntry, random_model
+    from hfee_amd.sampling import Sampler, SamplingParams
+    cfg = config_from_dict(cj)
+    model = random_model(cfg, seed=0, dtype="bfloat16", device="cuda:0", std=0.02)
+    spec = model.spec
+    matrices = [t for t in model.tensor_specs() if len(t.shape) == 2 and t.name != spec.embedding_name]
+    weight_bytes = 2 * sum(t.shape[0] * t.shape[1] for t in matrices)
+    layer_flops_a_token = 2 * sum(t.shape[0] * t.shape[1] for t in matrices)
+    attention_dims = 0          # (key size + value size) x heads, summed over the layers, as the kernels see them
+    for ls in spec.layers:
+        m = ls.mixer
+        if m.kind == "attention":
+            attention_dims += 2 * m.get("head_dim") * m.get("num_heads")
+        elif m.kind == "kv_attention":
+            attention_dims += (m.get("key_dim") + m.get("value_dim")) * m.get("num_heads")
+        elif m.kind == "latent_attention":
+            attention_dims += (2 * m.get("kv_rank") + m.get("rotated_dim")) * m.get("num_heads")
+    page_size, context = 16, 4096
+    engine = Engine(model, cache_tokens=batch * (PROMPT + steps + warmup + 4 * page_size) + PREFILL + page_size,
+                    page_size=page_size, max_requests=max(batch, 2), max_batch_tokens=PREFILL, num_positions=context)
+    sampler = Sampler(spec.vocab, engine.device, max_rows=max(batch, 2))
+    gen = torch.Generator().manual_seed(0)
+    best = None
+    for i in range(3):
+        prompt = torch.randint(0, spec.vocab, (PREFILL,), generator=gen).tolist()
+        engine.admit(("prefill", i))
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        engine.step([StepEntry(("prefill", i), prompt, [PREFILL - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        engine.release(("prefill", i))
+        best = dt if best is None else min(best, dt)
+    prefill_flops = PREFILL * layer_flops_a_token + 2.0 * attention_dims * PREFILL * (PREFILL + 1) / 2
+    sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=context)
+    params = SamplingParams.greedy(num_predict=-1, ignore_eos=True)
+    for i in range(batch):
+        sched.add(Request(("bench", i), torch.randint(0, spec.vocab, (PROMPT,), generator=gen).tolist(), params, seed=i))
+    while any(not r.decoding for r in list(sched.running) + list(sched.waiting)):
+        sched.step()
+    for _ in range(warmup):
+        sched.step()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        sched.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t) / steps
+    step_bytes = weight_bytes + batch * (PROMPT + warmup + steps / 2) * bytes_per_token(engine.groups, torch.bfloat16)
+    for r in list(sched.running):
+        sched.cancel(r.request_id)
+    while sched.has_work():
+        sched.step()
+    out = {"prefill_2048_tok_s": round(PREFILL / best, 1), "prefill_2048_ms": round(best * 1e3, 3),
+           "prefill_frac_of_matrix_peak": round(prefill_flops / best / BF16_PEAK, 4),
+           f"decode_b{batch}_tok_s": round(batch / dt, 1), f"decode_b{batch}_ms_per_step": round(dt * 1e3, 4),
+           "decode_frac_of_hbm_peak": round(step_bytes / dt / HBM_PEAK, 4),
+           "weight_gb": round(weight_bytes / 1e9, 3), "graph_replays": engine.graph_replays}
+    del sched, sampler, engine, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def vofezen_compare(args) -> dict:
+    import hfee_amd  # noqa: F401
+    layers = args.layers or 8
+    points = {}
+    for name, size in VOFEZEN_SIZES.items():
+        if args.vofezen_size not in (None, name):
+            continue
+        vof, llama = vofezen_configs(size, layers)
+        for design, cj in (("vofezen", vof), ("llama", llama)):
+            if args.vofezen_design not in ("both", design):
+                continue
+            print(f"[bench] {design} {name}, {layers} layers", file=sys.stderr, flush=True)
+            points[f"{design}_{name}"] = design_point(cj, args.batch, min(args.steps, 32), min(args.warmup, 4))
+    return {"metric": "Vofezen beside Llama at equal layer sizes: prefill of 2,048 tokens, decode at batch %d and "
+                      "1,024-token prompts (bf16, random weights)" % args.batch,
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": layers, "points": points}
+
+
 def main(argv=None) -> int:
     args = parse(argv)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.vofezen:
+        print(json.dumps(vofezen_compare(args)), flush=True)
+        return 0
     if args.yardsticks:
         import hfee_amd  # noqa: F401
         gbs, tflops = yardsticks()

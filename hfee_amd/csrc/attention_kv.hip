@@ -21,7 +21,8 @@ using namespace hfee;
 namespace {
 
 // ---------------------------------------------------------------- rotation + cache write
-// One workgroup a token.  q is rotated in place; k (rotated) and v (blended, if asked) go
+// A token's elements (pairs of q, elements of k and of v) are spread over the threads of
+// gridDim.y workgroups.  q is rotated in place; k (rotated) and v (blended, if asked) go
 // into the token's slot.  The rotated dims of a head are [rot_off, rot_off + 2 * half), pairs
 // (i, i + half); cos/sin tables [positions][half] carry the amplitude.
 template <typename T>
@@ -36,9 +37,10 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
   const int pos = positions[t];
   const float* c = cos_t + (int64_t)pos * half;
   const float* s = sin_t + (int64_t)pos * half;
+  const int first = blockIdx.y * blockDim.x + threadIdx.x, stride = gridDim.y * blockDim.x;
   if (q != nullptr) {
     T* qr = q + (int64_t)t * ldq;
-    for (int e = threadIdx.x; e < num_heads * half; e += blockDim.x) {
+    for (int e = first; e < num_heads * half; e += stride) {
       const int h = e / half, i = e - h * half;
       T* p = qr + (int64_t)h * q_dim + q_rot_off + i;
       const float a = to_float<T>(p[0]), b = to_float<T>(p[half]);
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
   const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
   const int slot = pos & (lay.page_size - 1);
   const T* kr = k + (int64_t)t * ldk;
-  for (int e = threadIdx.x; e < lay.kv_heads * lay.dk; e += blockDim.x) {
+  for (int e = first; e < lay.kv_heads * lay.dk; e += stride) {
     const int g = e / lay.dk, d = e - g * lay.dk;
     const int i = d - k_rot_off;
     float val;
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
   const T* vr = v + (int64_t)t * ldv;
   const int vw = lay.kv_heads * lay.dv;
   const float lam = v_first_mode == 2 ? to_float<T>(v_mix[0]) : 0.f;
-  for (int e = threadIdx.x; e < vw; e += blockDim.x) {
+  for (int e = first; e < vw; e += stride) {
     const int g = e / lay.dv, d = e - g * lay.dv;
     T val = vr[e];
     if (v_first_mode == 1) {
@@ -156,41 +158,59 @@ __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
 
 // ---------------------------------------------------------------- per-head product
 // out[t, h, o] = sum_i w[h][i][o] * x[t, h, i] for o < n_out (w stored [heads][n_in][n_out], so
-// that neighbouring threads read neighbouring weights), in ascending i; then `tail` elements
-// x[t, h, n_in ..] are copied behind them.  A workgroup takes one head and kTokens tokens.
-constexpr int kHeadLinearTokens = 8;
+// that neighbouring threads read neighbouring weights); then `tail` elements x[t, h, n_in ..]
+// are copied behind them.  A workgroup takes one head, kHeadLinearTokens tokens and 32 outputs;
+// its 256 threads are 8 slices of the inputs x 32 outputs, each slice summed in ascending i and
+// the slices added in their order: a token's result does not depend on the tokens beside it.
+constexpr int kHeadLinearTokens = 8, kHeadLinearOutputs = 32, kHeadLinearSlices = 8;
 
 template <typename T>
 __global__ __launch_bounds__(256) void head_linear_kernel(
     T* __restrict__ out, int64_t ldo, int64_t out_head_stride, const T* __restrict__ x, int64_t ldx,
     int64_t x_head_stride, const T* __restrict__ w, int n_in, int n_out, int tail, int n) {
-  extern __shared__ float xs[];      // [kTokens][n_in]
-  const int h = blockIdx.y, t0 = blockIdx.x * kHeadLinearTokens;
+  extern __shared__ float xs[];      // [kTokens][n_in], then [slices][kTokens][32] partial sums
+  float* part = xs + kHeadLinearTokens * n_in;
+  const int h = blockIdx.y, t0 = blockIdx.x * kHeadLinearTokens, o0 = blockIdx.z * kHeadLinearOutputs;
   const int count = min(kHeadLinearTokens, n - t0);
-  for (int e = threadIdx.x; e < count * n_in; e += blockDim.x) {
+  for (int e = threadIdx.x; e < kHeadLinearTokens * n_in; e += blockDim.x) {
     const int r = e / n_in, i = e - r * n_in;
-    xs[e] = to_float<T>(x[(int64_t)(t0 + r) * ldx + (int64_t)h * x_head_stride + i]);
+    xs[e] = r < count ? to_float<T>(x[(int64_t)(t0 + r) * ldx + (int64_t)h * x_head_stride + i]) : 0.f;
   }
   __syncthreads();
+  const int lane_o = threadIdx.x & (kHeadLinearOutputs - 1), slice = threadIdx.x / kHeadLinearOutputs;
+  const int o = o0 + lane_o;
+  const int per = (n_in + kHeadLinearSlices - 1) / kHeadLinearSlices;
+  const int i0 = slice * per, i1 = min(n_in, i0 + per);
   const T* wh = w + (int64_t)h * n_in * n_out;
-  for (int o = threadIdx.x; o < n_out; o += blockDim.x) {
-    float acc[kHeadLinearTokens];
+  float acc[kHeadLinearTokens];
 #pragma unroll
-    for (int r = 0; r < kHeadLinearTokens; ++r) acc[r] = 0.f;
-    for (int i = 0; i < n_in; ++i) {
+  for (int r = 0; r < kHeadLinearTokens; ++r) acc[r] = 0.f;
+  if (o < n_out) {
+#pragma unroll 4
+    for (int i = i0; i < i1; ++i) {
       const float wv = to_float<T>(wh[(int64_t)i * n_out + o]);
 #pragma unroll
       for (int r = 0; r < kHeadLinearTokens; ++r) acc[r] = fmaf(wv, xs[r * n_in + i], acc[r]);
     }
+  }
 #pragma unroll
-    for (int r = 0; r < kHeadLinearTokens; ++r)
-      if (r < count) out[(int64_t)(t0 + r) * ldo + (int64_t)h * out_head_stride + o] = from_float<T>(acc[r]);
+  for (int r = 0; r < kHeadLinearTokens; ++r) part[(slice * kHeadLinearTokens + r) * kHeadLinearOutputs + lane_o] = acc[r];
+  __syncthreads();
+  {
+    const int r = threadIdx.x / kHeadLinearOutputs;       // 8 tokens x 32 outputs = the workgroup's 256 threads
+    if (r < count && o < n_out) {
+      float sum = 0.f;
+#pragma unroll
+      for (int sl = 0; sl < kHeadLinearSlices; ++sl) sum += part[(sl * kHeadLinearTokens + r) * kHeadLinearOutputs + lane_o];
+      out[(int64_t)(t0 + r) * ldo + (int64_t)h * out_head_stride + o] = from_float<T>(sum);
+    }
   }
-  for (int e = threadIdx.x; e < count * tail; e += blockDim.x) {
-    const int r = e / tail, i = e - r * tail;
-    out[(int64_t)(t0 + r) * ldo + (int64_t)h * out_head_stride + n_out + i] =
-        x[(int64_t)(t0 + r) * ldx + (int64_t)h * x_head_stride + n_in + i];
-  }
+  if (blockIdx.z == 0)
+    for (int e = threadIdx.x; e < count * tail; e += blockDim.x) {
+      const int r = e / tail, i = e - r * tail;
+      out[(int64_t)(t0 + r) * ldo + (int64_t)h * out_head_stride + n_out + i] =
+          x[(int64_t)(t0 + r) * ldx + (int64_t)h * x_head_stride + n_in + i];
+    }
 }
 
 }  // namespace
@@ -221,8 +241,15 @@ HFEE_API int hfee_kv_write(void* q, int64_t ldq, int num_heads, int q_dim, int q
   } else {
     lay = KvLayout{};
   }
+  // few tokens: as many workgroups a token as its largest run of elements has blocks of 256 (at most 16)
+  int most = num_heads * half;
+  if (k != nullptr && kv_heads * dk > most) most = kv_heads * dk;
+  if (k != nullptr && kv_heads * dv > most) most = kv_heads * dv;
+  int parts = n >= 1024 ? 1 : (most + 255) / 256;
+  if (parts > 16) parts = 16;
+  if (parts < 1) parts = 1;
 #define LAUNCH(T)                                                                                                    \
-  kv_write_kernel<T><<<n, 256, 0, stream>>>((T*)q, ldq, num_heads, q_dim, q_rot_off, (const T*)k, ldk, k_rot_off,    \
+  kv_write_kernel<T><<<dim3(n, parts), 256, 0, stream>>>((T*)q, ldq, num_heads, q_dim, q_rot_off, (const T*)k, ldk, k_rot_off,    \
       (const T*)v, ldv, (T*)v_first, v_first_mode, (const T*)v_mix, positions, token_segment, block_tables,          \
       bt_stride, cos_t, sin_t, half, (T*)cache, lay)
   if (dtype == 0) LAUNCH(float);
@@ -267,10 +294,11 @@ HFEE_API int hfee_head_linear(void* out, int64_t ldo, int64_t out_head_stride, c
                               int tail, int n, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && heads > 0 && n_in > 0 && n_out > 0 && tail >= 0, "head_linear: bad sizes");
   if (n == 0) return 0;
-  HFEE_REQUIRE(heads <= 65535 && n_in <= 2048, "head_linear: at most 65535 heads and 2048 inputs a head");
+  HFEE_REQUIRE(heads <= 65535 && n_in <= 1536, "head_linear: at most 65535 heads and 1536 inputs a head");
   HFEE_REQUIRE(x_head_stride >= n_in + tail && out_head_stride >= n_out + tail, "head_linear: heads overlap");
-  dim3 grid((n + kHeadLinearTokens - 1) / kHeadLinearTokens, heads);
-  const size_t lds = (size_t)kHeadLinearTokens * n_in * sizeof(float);
+  HFEE_REQUIRE((n_out + kHeadLinearOutputs - 1) / kHeadLinearOutputs <= 65535, "head_linear: too many outputs a head");
+  dim3 grid((n + kHeadLinearTokens - 1) / kHeadLinearTokens, heads, (n_out + kHeadLinearOutputs - 1) / kHeadLinearOutputs);
+  const size_t lds = ((size_t)kHeadLinearTokens * n_in + kHeadLinearSlices * kHeadLinearTokens * kHeadLinearOutputs) * sizeof(float);
   if (dtype == 0)
     head_linear_kernel<float><<<grid, 256, lds, stream>>>((float*)out, ldo, out_head_stride, (const float*)x, ldx,
         x_head_stride, (const float*)w, n_in, n_out, tail, n);

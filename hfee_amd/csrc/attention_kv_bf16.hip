@@ -10,7 +10,8 @@
 // values of a value column are two loads of 8 bytes from the transposed values).
 //
 // Two meanings of the 16 rows (`mode`):
-//   0  a portion of a prompt: 16 consecutive tokens of one sequence, one head a wave;
+//   0  a portion of a prompt: up to four blocks of 16 consecutive tokens of one sequence (as many as
+//      the registers hold for the sizes), one head a wave;
 //   1  a single token: up to 16 query heads that share a key/value head; the keys may be
 //      split over several waves, whose partial results a second kernel joins.
 // The sink joins the denominator once, at the very end.
@@ -48,7 +49,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 // partial results of a split: [item][head][split][4 + DV] float32: maximum (base 2), sum, two unused, O
 constexpr int kPartial = 4 + DV;
 
-template <int MODE>
+// Row blocks of 16 that a wave of a prompt portion owns: the key and value operands of a tile
+// are loaded once and multiplied with every row block, so the more blocks the registers hold
+// (queries and output sums of a block: 4 (KSTEPS + VBLOCKS) registers a lane), the fewer bytes a
+// product costs.
+constexpr int kRegistersABlock = 4 * (KSTEPS + VBLOCKS);
+constexpr int PORTION_BLOCKS = kRegistersABlock <= 64 ? 4 : kRegistersABlock <= 128 ? 2 : 1;
+
+template <int MODE, int RB>
 __global__ __launch_bounds__(256) void attention_kv_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
     const bf16_t* __restrict__ cache, KvLayout lay, const int* __restrict__ items, int num_items,
@@ -66,34 +74,45 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
   const int row0 = items[item * 4 + 0], rows = items[item * 4 + 1], pos0 = items[item * 4 + 2];
   const int* bt = block_tables + (int64_t)items[item * 4 + 3] * bt_stride;
 
-  int token, head, pos, kvh;
-  bool valid;
+  // row r of block b: a token of the portion (mode 0), or a head of the key/value head's group (mode 1)
+  int token[RB], head[RB], pos[RB], kvh;
+  bool valid[RB];
   if (MODE == 0) {
-    const int rr = min(r, rows - 1);
-    token = row0 + rr; pos = pos0 + rr; head = unit; kvh = head / hpg; valid = r < rows;
+    kvh = unit / hpg;
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      const int rr = min(16 * b + r, rows - 1);
+      token[b] = row0 + rr; pos[b] = pos0 + rr; head[b] = unit; valid[b] = 16 * b + r < rows;
+    }
   } else {
     kvh = unit / groups16;
     const int in_group = (unit % groups16) * 16 + r;
-    valid = in_group < hpg;
-    token = row0; pos = pos0; head = kvh * hpg + min(in_group, hpg - 1);
+    valid[0] = in_group < hpg;
+    token[0] = row0; pos[0] = pos0; head[0] = kvh * hpg + min(in_group, hpg - 1);
   }
   const int max_pos = MODE == 0 ? pos0 + rows - 1 : pos0;
+  const int blocks = MODE == 0 ? (rows + 15) >> 4 : 1;       // row blocks that hold rows at all
 
   // the queries as the column operand: lane (r, g) holds dims 8g .. 8g+7 of every step of row r
-  Operand qop[KSTEPS];
-  {
-    const bf16_t* qr = q + (int64_t)token * ldq + (int64_t)head * DK + g * 8;
+  Operand qop[RB][KSTEPS];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const bf16_t* qr = q + (int64_t)token[b] * ldq + (int64_t)head[b] * DK + g * 8;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
-      if (s * 32 + g * 8 < DK) qop[s].u = *reinterpret_cast<const u32x4*>(qr + s * 32);
-      else qop[s].u = u32x4{0, 0, 0, 0};
+      if (s * 32 + g * 8 < DK) qop[b][s].u = *reinterpret_cast<const u32x4*>(qr + s * 32);
+      else qop[b][s].u = u32x4{0, 0, 0, 0};
     }
   }
 
-  f32x4 acc[VBLOCKS];
+  f32x4 acc[RB][VBLOCKS];
+  float m[RB], lsum[RB];
 #pragma unroll
-  for (int b = 0; b < VBLOCKS; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, lsum = 0.f;
+  for (int b = 0; b < RB; ++b) {
+    m[b] = -INFINITY; lsum[b] = 0.f;
+#pragma unroll
+    for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   const int ntiles = (max_pos >> 5) + 1;
   const int per_split = (ntiles + splits - 1) / splits;
@@ -103,112 +122,138 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
 
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     const int j0 = tile << 5;
-    f32x4 s[2];
+    // which row blocks see any key of this tile (the same answer in every lane)
+    bool live[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) live[b] = b < blocks && j0 <= pos0 + (MODE == 0 ? min(rows - 1, 16 * b + 15) : 0);
+    f32x4 s[RB][2];
     const bf16_t* vbase[2];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      const int jb = j0 + b * 16;
+    for (int kb = 0; kb < 2; ++kb) {
+      const int jb = j0 + kb * 16;
       const int page = bt[min(jb >> lay.page_shift, last_block)];
       const int slot0 = jb & slot_mask;
       const bf16_t* kr = cache + lay.key_offset(page, kvh, slot0 + r, g * 8);
-      vbase[b] = cache + lay.values_of(page, kvh) + slot0 + g * 4;
-      s[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+      vbase[kb] = cache + lay.values_of(page, kvh) + slot0 + g * 4;
+#pragma unroll
+      for (int b = 0; b < RB; ++b) s[b][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int st = 0; st < KSTEPS; ++st) {
         Operand kop;
         if (st * 32 + g * 8 < DK) kop.u = *reinterpret_cast<const u32x4*>(kr + st * 32);
         else kop.u = u32x4{0, 0, 0, 0};
-        s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qop[st].v, s[b], 0, 0, 0);
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+          if (live[b]) s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qop[b][st].v, s[b][kb], 0, 0, 0);
       }
     }
-    // scores of query r (this lane's column) against keys j0 + 16 b + 4 g + i
-    float tmax = -INFINITY;
+    // scores of query r (this lane's column) against keys j0 + 16 kb + 4 g + i
+    Operand pop[RB];
+    float alpha[RB];
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < RB; ++b) {
+      if (!live[b]) continue;
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = j0 + b * 16 + g * 4 + i;
-        const float v = key <= pos ? s[b][i] * scale_log2 : -INFINITY;
-        s[b][i] = v;
-        tmax = fmaxf(tmax, v);
-      }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m, tmax);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = exp2f(m - m_use);
-    m = m_new;
-    float psum = 0.f;
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+        for (int i = 0; i < 4; ++i) {
+          const int key = j0 + kb * 16 + g * 4 + i;
+          const float v = key <= pos[b] ? s[b][kb][i] * scale_log2 : -INFINITY;
+          s[b][kb][i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m[b], tmax);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      alpha[b] = exp2f(m[b] - m_use);
+      m[b] = m_new;
+      float psum = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = exp2f(s[b][i] - m_use);
-        s[b][i] = p;
-        psum += p;
-      }
-    lsum = lsum * alpha + psum;
-    Operand pop;
-    pop.u = u32x4{pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]), pack_bf16(s[1][0], s[1][1]),
-                  pack_bf16(s[1][2], s[1][3])};
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float p = exp2f(s[b][kb][i] - m_use);
+          s[b][kb][i] = p;
+          psum += p;
+        }
+      lsum[b] = lsum[b] * alpha[b] + psum;
+      pop[b].u = u32x4{pack_bf16(s[b][0][0], s[b][0][1]), pack_bf16(s[b][0][2], s[b][0][3]),
+                       pack_bf16(s[b][1][0], s[b][1][1]), pack_bf16(s[b][1][2], s[b][1][3])};
+    }
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) {
       Operand vop;
       const int64_t column = (int64_t)(vb * 16 + r) * lay.page_size;
       vop.h[0] = *reinterpret_cast<const u32x2*>(vbase[0] + column);
       vop.h[1] = *reinterpret_cast<const u32x2*>(vbase[1] + column);
-      acc[vb] = acc[vb] * alpha;
-      acc[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop.v, acc[vb], 0, 0, 0);
+#pragma unroll
+      for (int b = 0; b < RB; ++b) {
+        if (!live[b]) continue;
+        acc[b][vb] = acc[b][vb] * alpha[b];
+        acc[b][vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop[b].v, acc[b][vb], 0, 0, 0);
+      }
     }
   }
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
 
-  if (splits == 1) {
-    if (sinks != nullptr) {
-      const float sk = sinks[head] * kLog2e;
-      const float m_all = fmaxf(m, sk);
-      const float a = exp2f(m - m_all);
-      lsum = lsum * a + exp2f(sk - m_all);
 #pragma unroll
-      for (int vb = 0; vb < VBLOCKS; ++vb) acc[vb] = acc[vb] * a;
+  for (int b = 0; b < RB; ++b) {
+    if (b >= blocks) continue;
+    float l = lsum[b];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (splits == 1) {
+      float a = 1.f;
+      if (sinks != nullptr) {
+        const float sk = sinks[head[b]] * kLog2e;
+        const float m_all = fmaxf(m[b], sk);
+        a = exp2f(m[b] - m_all);
+        l = l * a + exp2f(sk - m_all);
+      }
+      if (!valid[b]) continue;
+      const float inv = a / l;
+      bf16_t* orow = out + (int64_t)token[b] * ld_out + (int64_t)head[b] * DV + g * 4;
+#pragma unroll
+      for (int vb = 0; vb < VBLOCKS; ++vb) {
+        const u32x2 w = {pack_bf16(acc[b][vb][0] * inv, acc[b][vb][1] * inv),
+                         pack_bf16(acc[b][vb][2] * inv, acc[b][vb][3] * inv)};
+        *reinterpret_cast<u32x2*>(orow + vb * 16) = w;
+      }
+    } else {
+      if (!valid[b]) continue;
+      float* pr = partial + (((int64_t)item * num_heads + head[b]) * splits + split) * kPartial;
+      if (g == 0) {
+        pr[0] = m[b];
+        pr[1] = l;
+      }
+#pragma unroll
+      for (int vb = 0; vb < VBLOCKS; ++vb)
+        *reinterpret_cast<f32x4*>(pr + 4 + vb * 16 + g * 4) = acc[b][vb];
     }
-    if (!valid) return;
-    const float inv = 1.0f / lsum;
-    bf16_t* orow = out + (int64_t)token * ld_out + (int64_t)head * DV + g * 4;
-#pragma unroll
-    for (int vb = 0; vb < VBLOCKS; ++vb) {
-      const u32x2 w = {pack_bf16(acc[vb][0] * inv, acc[vb][1] * inv), pack_bf16(acc[vb][2] * inv, acc[vb][3] * inv)};
-      *reinterpret_cast<u32x2*>(orow + vb * 16) = w;
-    }
-    return;
   }
-  if (!valid) return;
-  float* pr = partial + (((int64_t)item * num_heads + head) * splits + split) * kPartial;
-  if (g == 0) {
-    pr[0] = m;
-    pr[1] = lsum;
-  }
-#pragma unroll
-  for (int vb = 0; vb < VBLOCKS; ++vb)
-    *reinterpret_cast<f32x4*>(pr + 4 + vb * 16 + g * 4) = acc[vb];
 }
 
-// joins the splits of a single token's heads: one wave per (item, head), lanes over the value dims
+// joins the splits of a single token's heads: one wave per (item, head).  Lane sp holds split sp's
+// maximum and sum (at most 64 splits), the weights of the splits come from one reduction over the
+// wave, and the value dims are then summed over the splits in their order, lanes over the dims.
 __global__ __launch_bounds__(64) void attention_kv_join_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const int* __restrict__ items, const float* __restrict__ partial,
     int splits, int num_heads, const float* __restrict__ sinks) {
   const int item = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const float* pr = partial + ((int64_t)item * num_heads + head) * splits * kPartial;
-  float m = sinks != nullptr ? sinks[head] * kLog2e : -INFINITY;
-  for (int sp = 0; sp < splits; ++sp) m = fmaxf(m, pr[sp * kPartial]);
-  float lsum = sinks != nullptr ? exp2f(sinks[head] * kLog2e - m) : 0.f;
-  for (int sp = 0; sp < splits; ++sp) lsum += pr[sp * kPartial + 1] * exp2f(pr[sp * kPartial] - m);
   const int token = items[item * 4];
+  const float sk = sinks != nullptr ? sinks[head] * kLog2e : -INFINITY;
+  const float my_m = lane < splits ? pr[lane * kPartial] : -INFINITY;
+  const float my_l = lane < splits ? pr[lane * kPartial + 1] : 0.f;
+  const float m = fmaxf(wave_max(my_m), sk);
+  const float my_w = exp2f(my_m - m);               // (0 for a split without keys and for lanes beyond the splits)
+  const float lsum = wave_sum(my_l * my_w) + (sinks != nullptr ? exp2f(sk - m) : 0.f);
+  const float inv = 1.0f / lsum;
   for (int d = lane; d < DV; d += 64) {
     float o = 0.f;
-    for (int sp = 0; sp < splits; ++sp) o += pr[sp * kPartial + 4 + d] * exp2f(pr[sp * kPartial] - m);
-    out[(int64_t)token * ld_out + (int64_t)head * DV + d] = float_to_bf16(o / lsum);
+    for (int sp = 0; sp < splits; ++sp) o = fmaf(pr[sp * kPartial + 4 + d], __shfl(my_w, sp, 64), o);
+    out[(int64_t)token * ld_out + (int64_t)head * DV + d] = float_to_bf16(o * inv);
   }
 }
 
@@ -218,14 +263,16 @@ HFEE_DEFINE_LAST_ERROR
 
 HFEE_API int hfee_attention_kv_bf16_dk() { return DK; }
 HFEE_API int hfee_attention_kv_bf16_dv() { return DV; }
+// the most rows of an item of mode 0
+HFEE_API int hfee_attention_kv_bf16_rows() { return 16 * PORTION_BLOCKS; }
 
 // float32 words of `partial` that `splits` > 1 need for `num_items` single tokens
 HFEE_API int64_t hfee_attention_kv_bf16_partial(int num_items, int num_heads, int splits) {
   return splits > 1 ? (int64_t)num_items * num_heads * splits * kPartial : 0;
 }
 
-// items: [num_items][4] int32 on the device: first row, rows (1..16; 1 in mode 1), first
-// position, block-table row.
+// items: [num_items][4] int32 on the device: first row, rows (1..hfee_attention_kv_bf16_rows() in
+// mode 0; 1 in mode 1), first position, block-table row.
 HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
                                     const int* items, int num_items, int mode, const int* block_tables,
                                     int bt_stride, int num_heads, int kv_heads, int page_size, float scale,
@@ -240,7 +287,7 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
   HFEE_REQUIRE(ldq >= (int64_t)num_heads * DK && ld_out >= (int64_t)num_heads * DV, "attention_kv_bf16: q/out row too short");
   HFEE_REQUIRE(ldq % 8 == 0 && ld_out % 4 == 0 && (uintptr_t)q % 16 == 0 && (uintptr_t)out % 8 == 0 &&
                (uintptr_t)cache % 16 == 0, "attention_kv_bf16: q, out and the cache must be aligned for vector access");
-  HFEE_REQUIRE(splits >= 1 && (splits == 1 || mode == 1), "attention_kv_bf16: only single tokens split their keys");
+  HFEE_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || mode == 1), "attention_kv_bf16: only single tokens split their keys, into at most 64");
   HFEE_REQUIRE(splits == 1 || (partial != nullptr &&
                partial_words >= hfee_attention_kv_bf16_partial(num_items, num_heads, splits)),
                "attention_kv_bf16: the partial results need more room");
@@ -253,10 +300,10 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
   HFEE_REQUIRE(blocks <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
   const float scale_log2 = scale * kLog2e;
   if (mode == 0)
-    attention_kv_kernel<0><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
+    attention_kv_kernel<0, PORTION_BLOCKS><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
         (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scale_log2, sinks, partial, 1);
   else
-    attention_kv_kernel<1><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
+    attention_kv_kernel<1, 1><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
         (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scale_log2, sinks, partial, splits);
   HFEE_CHECK_LAUNCH("attention_kv_bf16");
   if (splits > 1) {

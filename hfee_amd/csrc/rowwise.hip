@@ -60,6 +60,66 @@ __global__ __launch_bounds__(256) void norm_add_kernel(
     nr[j] = from_float<TN>(xr[j] * inv2 * weight_at<TW>(w2, j, offset));
 }
 
+// The same for float32 y, bias and weights and rows of a multiple of four that fit the workgroup's
+// registers (4 NV values a thread): everything a row needs is asked for at once, so that the row
+// costs one trip to memory, two sums over the workgroup and the stores.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <typename TN> __device__ __forceinline__ void store4(TN* p, f32x4_t v);
+template <> __device__ __forceinline__ void store4<float>(float* p, f32x4_t v) { *reinterpret_cast<f32x4_t*>(p) = v; }
+template <> __device__ __forceinline__ void store4<bf16_t>(bf16_t* p, f32x4_t v) {
+  typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+  const u32x2_t w = {(uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16),
+                     (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16)};
+  *reinterpret_cast<u32x2_t*>(p) = w;
+}
+
+template <typename TN, int NV>
+__global__ __launch_bounds__(1024) void norm_add_rows_kernel(
+    float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ bias, const float* __restrict__ w,
+    float eps, TN* __restrict__ next, const float* __restrict__ w2, float eps2, int d) {
+  __shared__ float scratch[16];
+  const int64_t r = blockIdx.x;
+  f32x4_t yv[NV], xv[NV], wv[NV], w2v[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int j = (k * blockDim.x + threadIdx.x) * 4;
+    const bool in = j < d;
+    const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+    yv[k] = in ? *reinterpret_cast<const f32x4_t*>(y + r * d + j) : zero;
+    if (in && bias != nullptr) yv[k] += *reinterpret_cast<const f32x4_t*>(bias + j);
+    xv[k] = in ? *reinterpret_cast<const f32x4_t*>(x + r * d + j) : zero;
+    wv[k] = in ? *reinterpret_cast<const f32x4_t*>(w + j) : zero;
+    w2v[k] = in && next != nullptr ? *reinterpret_cast<const f32x4_t*>(w2 + j) : zero;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss = fmaf(yv[k][i], yv[k][i], ss);
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int j = (k * blockDim.x + threadIdx.x) * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      xv[k][i] += yv[k][i] * inv * wv[k][i];
+      ss2 = fmaf(xv[k][i], xv[k][i], ss2);
+    }
+    if (j < d) *reinterpret_cast<f32x4_t*>(x + r * d + j) = xv[k];
+  }
+  if (next == nullptr) return;
+  ss2 = block_sum(ss2, scratch);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)d + eps2);
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int j = (k * blockDim.x + threadIdx.x) * 4;
+    if (j < d) store4<TN>(next + r * d + j, xv[k] * inv2 * w2v[k]);
+  }
+}
+
 template <typename T>
 __global__ void bias_act_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ in, int64_t ldi,
                                 const T* __restrict__ bias, int width, int act) {
@@ -99,6 +159,26 @@ HFEE_API int hfee_norm_add(float* x, const void* y, int y_dtype, const void* bia
   HFEE_REQUIRE(eps >= 0.f && eps2 >= 0.f, "norm_add: eps must not be negative");
   HFEE_REQUIRE(next == nullptr || w2 != nullptr, "norm_add: the following norm needs its weight");
   if (n == 0) return 0;
+  const bool aligned = ((uintptr_t)x | (uintptr_t)y | (uintptr_t)bias | (uintptr_t)w | (uintptr_t)w2) % 16 == 0 &&
+                       (uintptr_t)next % 8 == 0;
+  if (offset == 0.f && y_dtype == 0 && (bias == nullptr || bias_dtype == 0) && w_dtype == 0 && d % 4 == 0 && d <= 16384 &&
+      aligned) {
+    const int quads = d / 4;
+    const int nv = quads <= 1024 ? 1 : quads <= 2048 ? 2 : 4;
+    int threads = ((quads + nv - 1) / nv + 63) / 64 * 64;
+    if (threads > 1024) threads = 1024;
+#define ROWS(TN, NV)                                                                                                  \
+  norm_add_rows_kernel<TN, NV><<<n, threads, 0, stream>>>(x, (const float*)y, (const float*)bias, (const float*)w, eps, \
+      (TN*)next, (const float*)w2, eps2, d)
+    if (next_dtype == 1 && next != nullptr) {
+      if (nv == 1) ROWS(bf16_t, 1); else if (nv == 2) ROWS(bf16_t, 2); else ROWS(bf16_t, 4);
+    } else {
+      if (nv == 1) ROWS(float, 1); else if (nv == 2) ROWS(float, 2); else ROWS(float, 4);
+    }
+#undef ROWS
+    HFEE_CHECK_LAUNCH("norm_add");
+    return 0;
+  }
   const int code = (y_dtype & 1) | ((bias_dtype & 1) << 1) | ((w_dtype & 1) << 2) | ((next_dtype & 1) << 3);
 #define CASE(c, TY, TB, TW, TN)                                                                                      \
   case c:                                                                                                            \

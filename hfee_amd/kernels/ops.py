@@ -873,6 +873,11 @@ def attention_kv_sizes_fit(dk: int, dv: int) -> bool:
     return dk % 16 == 0 and dv % 16 == 0 and 16 <= dk <= build.ATTENTION_KV_MOST[0] and 16 <= dv <= build.ATTENTION_KV_MOST[1]
 
 
+def attention_kv_rows(dk: int, dv: int) -> int:
+    """The most rows that an item of `attention_kv_bf16`'s mode 0 may hold for these sizes."""
+    return int(lib.attention_kv_bf16(dk, dv).raw("hfee_attention_kv_bf16_rows")())
+
+
 def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: int) -> int:
     return num_items * num_heads * splits * (4 + dv) if splits > 1 else 0
 
@@ -880,7 +885,7 @@ def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: 
 def attention_kv_bf16(out, q, cache_layer, items, mode: int, block_tables, num_heads: int, kv_heads: int, dk: int,
                       dv: int, page_size: int, scale: float, sinks=None, partial=None, splits: int = 1):
     """Matrix-core attention, bfloat16.  items: int32 [count, 4] on the device (first row, rows,
-    first position, block-table row).  mode 0: an item is up to 16 consecutive tokens of a portion;
+    first position, block-table row).  mode 0: an item is up to `attention_kv_rows` consecutive tokens of a portion;
     mode 1: an item is a single token (rows = 1), whose keys may be split over `splits` waves that
     leave partial results in `partial` (float32, `attention_kv_partial_words`) for a joining kernel."""
     _gpu(out, q, cache_layer, items, block_tables, sinks, partial)

@@ -36,28 +36,25 @@ from ..kernels import ops
 from ..weights.spec import TensorSpec
 from .base import LazyNorm, Mixer, lookup, register_mixer
 
-_ROWS = 16             # query rows of a matrix-core tile
+_ROWS = 16             # rows of a matrix-core tile: the heads of a key/value head that one wave takes for a single token
 _KEY_TILE = 32         # keys of a step of the matrix-core kernels
 _WAVES_WANTED = 2048   # single tokens split their keys until about this many waves run
 _MOST_SPLITS = 64
 _LAYOUT = "keys by slot, then values by dimension"
 
 
-def plan_items(plan) -> None:
+def plan_items(plan, rows: int) -> None:
     """The step's work for the matrix-core kernels, once a step whichever layers ask: portions in
-    tiles of 16 rows, single tokens one by one (first row, rows, first position, block-table row)."""
-    if "attention_kv.portions" in plan.arrays:
-        return
-    portions, singles = [], []
-    for s, seg in enumerate(plan.segments):
-        if seg.length == 1:
-            singles.append((seg.row0, 1, seg.start, s))
-        else:
-            for off in range(0, seg.length, _ROWS):
-                portions.append((seg.row0 + off, min(_ROWS, seg.length - off), seg.start + off, s))
-    plan.add("attention_kv.portions", np.asarray(portions, dtype=np.int32).reshape(-1, 4))
-    plan.add("attention_kv.singles", np.asarray(singles, dtype=np.int32).reshape(-1, 4))
-    plan.host["attention_kv.single_max_position"] = max([p for _, _, p, _ in singles], default=0)
+    tiles of `rows` rows (the most that the kernels of a layer's sizes take), single tokens one by
+    one (first row, rows, first position, block-table row)."""
+    if f"attention_kv.portions.{rows}" not in plan.arrays:
+        portions = [(seg.row0 + off, min(rows, seg.length - off), seg.start + off, s)
+                    for s, seg in enumerate(plan.segments) if seg.length > 1 for off in range(0, seg.length, rows)]
+        plan.add(f"attention_kv.portions.{rows}", np.asarray(portions, dtype=np.int32).reshape(-1, 4))
+    if "attention_kv.singles" not in plan.arrays:
+        singles = [(seg.row0, 1, seg.start, s) for s, seg in enumerate(plan.segments) if seg.length == 1]
+        plan.add("attention_kv.singles", np.asarray(singles, dtype=np.int32).reshape(-1, 4))
+        plan.host["attention_kv.single_max_position"] = max([p for _, _, p, _ in singles], default=0)
 
 
 def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks, matrix: bool) -> None:
@@ -65,7 +62,8 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
         ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
                                ctx.page_size, scale, sinks)
         return
-    portions, singles = ctx.extra["attention_kv.portions"], ctx.extra["attention_kv.singles"]
+    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv)}"]
+    singles = ctx.extra["attention_kv.singles"]
     if portions.shape[0]:
         ops.attention_kv_bf16(out, q, cache, portions, 0, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks)
     count = singles.shape[0]
@@ -81,6 +79,24 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
                                          torch.float32)
         ops.attention_kv_bf16(out, q, cache, singles, 1, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks,
                               partial=partial, splits=splits)
+
+
+def tiles_of(dtype, *weights):
+    """The weights' second copies in tiles, which the products of up to 64 rows stream (None where
+    the engine is not bfloat16, a width is no multiple of 8, or the memory has no room)."""
+    if dtype != torch.bfloat16 or any(w.shape[0] % 8 or w.shape[1] % 8 for w in weights):
+        return (None,) * len(weights)
+    return ops.tile_weights_if_room(*weights) or (None,) * len(weights)
+
+
+def product(ctx, out, x, weight, tiles=None) -> None:
+    """out = x @ weight.T: up to 64 rows stream the weight's tiles, more go through the tiled kernels."""
+    n = x.shape[0]
+    if tiles is not None and n <= ops.SKINNY_MAX_ROWS:
+        ops.linear_fused(out, x, tiles, "f32" if out.dtype == torch.float32 else "bf16",
+                         **ctx.workspace.product_scratch(n, tiles))
+    else:
+        ops.linear(out, x, weight, **ctx.workspace.split_scratch(n, weight))
 
 
 class _KvMixer(Mixer):
@@ -100,7 +116,7 @@ class _KvMixer(Mixer):
 
     def plan(self, plan):
         if self.matrix:
-            plan_items(plan)
+            plan_items(plan, ops.attention_kv_rows(*self.kernel_sizes))
 
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
         y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
@@ -134,6 +150,7 @@ class KvAttention(_KvMixer):
                                             sink="sinks", value_blend="value_blend"))
         self.q_width, self.k_width, self.v_width = self.num_heads * self.dk, self.kv_heads * self.dk, self.kv_heads * self.dv
         self.out_width = self.num_heads * self.dv
+        self.kernel_sizes = (self.dk, self.dv)
         self.matrix = self._matrix(self.dk, self.dv, self.q_width + self.k_width + self.v_width, self.out_width)
 
     def tensor_specs(self):
@@ -153,6 +170,7 @@ class KvAttention(_KvMixer):
         self.sinks = tensors.pop(n["sink"]).to(torch.float32).contiguous() if self.has_sink else None
         t = tensors.pop(n["value_blend"], None)
         self.blend_weight = t.reshape(1).to(self.dtype).contiguous() if (t is not None and self.blend == "mix") else None
+        self.w_qkv_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_qkv, self.w_o)
 
     def cache_spec(self):
         return CacheNeed("full", (self.kv_heads, self.dk + self.dv), 0, layout=_LAYOUT)
@@ -172,7 +190,7 @@ class KvAttention(_KvMixer):
         qkv = ctx.rows("kv_attention.qkv", self.q_width + self.k_width + self.v_width)
         q = qkv[:, :self.q_width]
         if writes_cache:
-            ops.linear(qkv, hn, self.w_qkv, **ctx.workspace.split_scratch(n, self.w_qkv))
+            product(ctx, qkv, hn, self.w_qkv, self.w_qkv_tiles)
             k = qkv[:, self.q_width:self.q_width + self.k_width]
             v = qkv[:, self.q_width + self.k_width:]
         else:       # this run of the layer reads keys and values that another run wrote
@@ -186,7 +204,7 @@ class KvAttention(_KvMixer):
                      v_mix=self.blend_weight)
         att = ctx.rows("kv_attention.out", self.out_width)
         attend(ctx, att, q, cache, tables, H, G, dk, dv, self.scale, self.sinks, self.matrix)
-        ops.linear(out, att, self.w_o, **ctx.workspace.split_scratch(n, self.w_o))
+        product(ctx, out, att, self.w_o, self.w_o_tiles)
 
 
 @register_mixer("latent_attention")
@@ -209,6 +227,7 @@ class LatentAttention(_KvMixer):
                                             v_up="v_b_proj.weight", o="o_proj.weight"))
         # the absorbed form: one key/value head, keys [latent | rotated part], values the latent
         self.dk_abs, self.dv_abs = self.kv_rank + self.rotated, self.kv_rank
+        self.kernel_sizes = (self.dk_abs, self.dv_abs)
         self.down_width = self.q_rank + self.kv_rank + self.rotated
         self.matrix = (self._matrix(self.dk_abs, self.dv_abs, self.num_heads * self.dk_abs, self.num_heads * self.dv_abs)
                        and self.down_width % 8 == 0 and self.q_rank % 8 == 0)
@@ -235,6 +254,7 @@ class LatentAttention(_KvMixer):
         self.w_k_absorb = tensors.pop(n["k_up"]).view(H, self.plain, self.kv_rank).contiguous()
         self.w_v_expand = tensors.pop(n["v_up"]).view(H, self.dv, self.kv_rank).transpose(1, 2).contiguous()
         self.w_o = tensors.pop(n["o"]).contiguous()
+        self.w_down_tiles, self.w_q_up_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_down, self.w_q_up, self.w_o)
 
     def cache_spec(self):
         return CacheNeed("full", (1, self.dk_abs + self.dv_abs), 0, layout=_LAYOUT)
@@ -254,13 +274,13 @@ class LatentAttention(_KvMixer):
         cos, sin = (pos.cos, pos.sin) if pos else (None, None)
         down = ctx.rows("latent.down", self.down_width)
         if writes_cache:
-            ops.linear(down, hn, self.w_down, **ctx.workspace.split_scratch(n, self.w_down))
+            product(ctx, down, hn, self.w_down, self.w_down_tiles)
         else:
             ops.linear(down[:, :self.q_rank], hn, self.w_down[:self.q_rank])
         cq = ctx.rows("latent.q_latent", self.q_rank)
         ops.rmsnorm_cols(cq, down[:, :self.q_rank], self.q_norm, self.eps)
         q = ctx.rows("latent.q", H * (Dn + Dr))
-        ops.linear(q, cq, self.w_q_up, **ctx.workspace.split_scratch(n, self.w_q_up))
+        product(ctx, q, cq, self.w_q_up, self.w_q_up_tiles)
         qa = ctx.rows("latent.q_absorbed", H * dk)
         ops.head_linear(qa, q, self.w_k_absorb, H, Dn, R, tail=Dr)
         k = v = None
@@ -274,4 +294,4 @@ class LatentAttention(_KvMixer):
         attend(ctx, att, qa, cache, tables, H, 1, dk, dv, self.scale, None, self.matrix)
         heads_out = ctx.rows("latent.values", H * self.dv)
         ops.head_linear(heads_out, att, self.w_v_expand, H, R, self.dv)
-        ops.linear(out, heads_out, self.w_o, **ctx.workspace.split_scratch(n, self.w_o))
+        product(ctx, out, heads_out, self.w_o, self.w_o_tiles)

@@ -133,15 +133,26 @@ class DenseMLP(FeedForward):
         self.w_up, self.w_down = tensors.pop(n["up"]).contiguous(), tensors.pop(n["down"]).contiguous()
         self.up_bias = tensors.pop(n["up_bias"]).to(self.dtype).contiguous() if self.has_bias else None
         self.output_bias = tensors.pop(n["down_bias"]).to(torch.float32).contiguous() if self.has_bias else None
+        # a second copy in tiles for steps of up to 64 rows, whose products stream the weights
+        self.w_up_tiles = self.w_down_tiles = None
+        if self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.intermediate % 8 == 0:
+            self.w_up_tiles, self.w_down_tiles = ops.tile_weights_if_room(self.w_up, self.w_down) or (None, None)
+
+    def _product(self, ctx, out, x, weight, tiles):
+        n = x.shape[0]
+        if tiles is not None and n <= ops.SKINNY_MAX_ROWS:
+            ops.linear_fused(out, x, tiles, "f32" if out.dtype == torch.float32 else "bf16",
+                             **ctx.workspace.product_scratch(n, tiles))
+        else:
+            ops.linear(out, x, weight, **ctx.workspace.split_scratch(n, weight))
 
     def forward_into(self, ctx, out, h):
         """out (float32 [n, hidden]) = down(activation(up(h) + b_up)); `output_bias` is not added."""
-        n = ctx.n
         hn = h.tensor() if isinstance(h, LazyNorm) else h
         act = ctx.rows("dense_mlp.act", self.intermediate)
-        ops.linear(act, hn, self.w_up, **ctx.workspace.split_scratch(n, self.w_up))
+        self._product(ctx, act, hn, self.w_up, self.w_up_tiles)
         ops.bias_act(act, act, self.up_bias, self.activation)
-        ops.linear(out, act, self.w_down, **ctx.workspace.split_scratch(n, self.w_down))
+        self._product(ctx, out, act, self.w_down, self.w_down_tiles)
 
     def forward_add(self, ctx, x, h):
         y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)

@@ -135,10 +135,10 @@ def test_attention_kernels(dtype, H, G, dk, dv):
     assert vu.rel(out.double().cpu(), no_sink) < tol
     if dtype == "float32" or not ops.attention_kv_sizes_fit(dk, dv):
         return
-    items0, row = [], 0
+    items0, row, most = [], 0, ops.attention_kv_rows(dk, dv)
     for s, (st, ln) in enumerate(zip(starts, lengths)):
         if ln > 1:
-            items0 += [(row + off, min(16, ln - off), st + off, s) for off in range(0, ln, 16)]
+            items0 += [(row + off, min(most, ln - off), st + off, s) for off in range(0, ln, most)]
         row += ln
     items1 = [(64, 1, 600, 2), (65, 1, 15, 3)]
     for sinks, ref in ((d_sink, want), (None, no_sink)):
