@@ -46,6 +46,50 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return (uint32_t)float_to_bf16(a) | ((uint32_t)float_to_bf16(b) << 16);
 }
 
+// The weights of one row block against a tile's 32 keys, in place in the score registers, and as the
+// column operand of the value product.  The exponentials are taken against a reference that lags
+// the running maximum: the sums are rescaled only when a maximum has moved by more than 2^8 (the
+// quotient at the end does not depend on the reference), so most tiles cost no pass over the
+// output sums.  Keys beyond the row's own position weigh nothing; `masked` says whether the tile
+// has any (the same answer in every lane).
+__device__ __forceinline__ void weigh_tile(f32x4 (&s)[2], float& reference, float& lsum, f32x4 (&acc)[VBLOCKS],
+                                           Operand& pop, int j0, int g, int pos, float scale_log2, bool masked) {
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float v = s[kb][i] * scale_log2;
+      if (masked && j0 + kb * 16 + g * 4 + i > pos) v = -INFINITY;
+      s[kb][i] = v;
+      tmax = fmaxf(tmax, v);
+    }
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+  if (__builtin_amdgcn_ballot_w64(tmax > reference + 8.0f) != 0) {      // (-inf + 8 = -inf: the first tile always)
+    const float moved = fmaxf(reference, tmax);
+    const float use = moved == -INFINITY ? 0.f : moved;
+    const float alpha = exp2f(reference - use);
+    reference = moved;
+    lsum *= alpha;
+#pragma unroll
+    for (int vb = 0; vb < VBLOCKS; ++vb) acc[vb] = acc[vb] * alpha;
+  }
+  const float use = reference == -INFINITY ? 0.f : reference;
+  float psum = 0.f;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p = exp2f(s[kb][i] - use);
+      s[kb][i] = p;
+      psum += p;
+    }
+  lsum += psum;
+  pop.u = u32x4{pack_bf16(s[0][0], s[0][1]), pack_bf16(s[0][2], s[0][3]), pack_bf16(s[1][0], s[1][1]),
+                pack_bf16(s[1][2], s[1][3])};
+}
+
 // partial results of a split: [item][head][split][4 + DV] float32: maximum (base 2), sum, two unused, O
 constexpr int kPartial = 4 + DV;
 
@@ -54,7 +98,18 @@ constexpr int kPartial = 4 + DV;
 // (queries and output sums of a block: 4 (KSTEPS + VBLOCKS) registers a lane), the fewer bytes a
 // product costs.
 constexpr int kRegistersABlock = 4 * (KSTEPS + VBLOCKS);
-constexpr int PORTION_BLOCKS = kRegistersABlock <= 64 ? 4 : kRegistersABlock <= 128 ? 2 : 1;
+#ifdef HFEE_KV_BLOCKS
+constexpr int PORTION_BLOCKS = HFEE_KV_BLOCKS;
+#else
+constexpr int PORTION_BLOCKS = kRegistersABlock <= 64 ? 2 : 1;
+#endif
+// The keys of the next tile are asked for while the weights of this one are made (a second set of
+// key operands: 8 KSTEPS registers a lane), where the registers allow it.
+#ifdef HFEE_KV_PIPE
+constexpr bool PIPE = HFEE_KV_PIPE;
+#else
+constexpr bool PIPE = 8 * KSTEPS + 4 * VBLOCKS <= 160;
+#endif
 
 template <int MODE, int RB>
 __global__ __launch_bounds__(256) void attention_kv_kernel(
@@ -120,79 +175,102 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
   const int last_block = max_pos >> lay.page_shift;
   const int slot_mask = lay.page_size - 1;
 
+  // the key operands of a tile: lane (r, g) holds dims 8g .. 8g+7 of every step of key r of each of the
+  // tile's two blocks of 16 keys; `values` gets where the lane's value columns of the two blocks begin
+  auto load_keys = [&](int tile, Operand (&kop)[2][PIPE ? KSTEPS : 1], const bf16_t* (&values)[2]) {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int jb = (tile << 5) + kb * 16;
+      const int page = bt[min(jb >> lay.page_shift, last_block)];
+      const int slot0 = jb & slot_mask;
+      const bf16_t* kr = cache + lay.key_offset(page, kvh, slot0 + r, g * 8);
+      values[kb] = cache + lay.values_of(page, kvh) + slot0 + g * 4;
+#pragma unroll
+      for (int st = 0; st < (PIPE ? KSTEPS : 1); ++st) {
+        if (st * 32 + g * 8 < DK) kop[kb][st].u = *reinterpret_cast<const u32x4*>(kr + st * 32);
+        else kop[kb][st].u = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  // (without the second set, a key operand lives from its load to its products only)
+  auto load_keys_of_block = [&](int tile, int kb, int st, const bf16_t*& values) {
+    const int jb = (tile << 5) + kb * 16;
+    const int page = bt[min(jb >> lay.page_shift, last_block)];
+    const int slot0 = jb & slot_mask;
+    values = cache + lay.values_of(page, kvh) + slot0 + g * 4;
+    Operand one;
+    if (st * 32 + g * 8 < DK) one.u = *reinterpret_cast<const u32x4*>(cache + lay.key_offset(page, kvh, slot0 + r, g * 8) + st * 32);
+    else one.u = u32x4{0, 0, 0, 0};
+    return one;
+  };
+  Operand kop[2][PIPE ? KSTEPS : 1];
+  const bf16_t* vnext[2];
+  if constexpr (PIPE) {
+    if (tile_begin < tile_end) load_keys(tile_begin, kop, vnext);
+  }
+
   for (int tile = tile_begin; tile < tile_end; ++tile) {
     const int j0 = tile << 5;
     // which row blocks see any key of this tile (the same answer in every lane)
     bool live[RB];
 #pragma unroll
-    for (int b = 0; b < RB; ++b) live[b] = b < blocks && j0 <= pos0 + (MODE == 0 ? min(rows - 1, 16 * b + 15) : 0);
+    for (int b = 0; b < RB; ++b)
+      live[b] = MODE == 1 || (b < blocks && j0 <= pos0 + min(rows - 1, 16 * b + 15));
     f32x4 s[RB][2];
     const bf16_t* vbase[2];
+    if constexpr (PIPE) {
+      vbase[0] = vnext[0];
+      vbase[1] = vnext[1];
+    }
+    Operand vop[PIPE ? VBLOCKS : 1];
+    if constexpr (PIPE) {
+#pragma unroll
+      for (int vb = 0; vb < VBLOCKS; ++vb) {
+        const int64_t column = (int64_t)(vb * 16 + r) * lay.page_size;
+        vop[vb].h[0] = *reinterpret_cast<const u32x2*>(vbase[0] + column);
+        vop[vb].h[1] = *reinterpret_cast<const u32x2*>(vbase[1] + column);
+      }
+    }
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
-      const int jb = j0 + kb * 16;
-      const int page = bt[min(jb >> lay.page_shift, last_block)];
-      const int slot0 = jb & slot_mask;
-      const bf16_t* kr = cache + lay.key_offset(page, kvh, slot0 + r, g * 8);
-      vbase[kb] = cache + lay.values_of(page, kvh) + slot0 + g * 4;
 #pragma unroll
       for (int b = 0; b < RB; ++b) s[b][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int st = 0; st < KSTEPS; ++st) {
-        Operand kop;
-        if (st * 32 + g * 8 < DK) kop.u = *reinterpret_cast<const u32x4*>(kr + st * 32);
-        else kop.u = u32x4{0, 0, 0, 0};
+        Operand now;
+        if constexpr (PIPE) now = kop[kb][st];
+        else now = load_keys_of_block(tile, kb, st, vbase[kb]);
 #pragma unroll
         for (int b = 0; b < RB; ++b)
-          if (live[b]) s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qop[b][st].v, s[b][kb], 0, 0, 0);
+          if (live[b]) s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(now.v, qop[b][st].v, s[b][kb], 0, 0, 0);
       }
+    }
+    if constexpr (PIPE) {
+      if (tile + 1 < tile_end) load_keys(tile + 1, kop, vnext);
     }
     // scores of query r (this lane's column) against keys j0 + 16 kb + 4 g + i
     Operand pop[RB];
-    float alpha[RB];
 #pragma unroll
     for (int b = 0; b < RB; ++b) {
       if (!live[b]) continue;
-      float tmax = -INFINITY;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = j0 + kb * 16 + g * 4 + i;
-          const float v = key <= pos[b] ? s[b][kb][i] * scale_log2 : -INFINITY;
-          s[b][kb][i] = v;
-          tmax = fmaxf(tmax, v);
-        }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m[b], tmax);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      alpha[b] = exp2f(m[b] - m_use);
-      m[b] = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float p = exp2f(s[b][kb][i] - m_use);
-          s[b][kb][i] = p;
-          psum += p;
-        }
-      lsum[b] = lsum[b] * alpha[b] + psum;
-      pop[b].u = u32x4{pack_bf16(s[b][0][0], s[b][0][1]), pack_bf16(s[b][0][2], s[b][0][3]),
-                       pack_bf16(s[b][1][0], s[b][1][1]), pack_bf16(s[b][1][2], s[b][1][3])};
+      // (the smallest position of the block's rows: a tile that ends at or before it hides no key)
+      const bool masked = j0 + 31 > (MODE == 0 ? pos0 + min(rows - 1, 16 * b) : pos0);
+      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, pos[b], scale_log2, masked);
     }
 #pragma unroll
     for (int vb = 0; vb < VBLOCKS; ++vb) {
-      Operand vop;
-      const int64_t column = (int64_t)(vb * 16 + r) * lay.page_size;
-      vop.h[0] = *reinterpret_cast<const u32x2*>(vbase[0] + column);
-      vop.h[1] = *reinterpret_cast<const u32x2*>(vbase[1] + column);
+      Operand values;
+      if constexpr (PIPE) {
+        values = vop[vb];
+      } else {
+        const int64_t column = (int64_t)(vb * 16 + r) * lay.page_size;
+        values.h[0] = *reinterpret_cast<const u32x2*>(vbase[0] + column);
+        values.h[1] = *reinterpret_cast<const u32x2*>(vbase[1] + column);
+      }
 #pragma unroll
       for (int b = 0; b < RB; ++b) {
         if (!live[b]) continue;
-        acc[b][vb] = acc[b][vb] * alpha[b];
-        acc[b][vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop[b].v, acc[b][vb], 0, 0, 0);
+        acc[b][vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(values.v, pop[b].v, acc[b][vb], 0, 0, 0);
       }
     }
   }
@@ -234,6 +312,204 @@ __global__ __launch_bounds__(256) void attention_kv_kernel(
   }
 }
 
+// Prompt portions where four query heads (or a multiple) share a key/value head: the four waves of
+// a workgroup are four heads of one group over the same rows, and every key tile comes from
+// memory once for all of them, into LDS (two stages: the next tile is on its way while this one is
+// multiplied; rows of keys padded by 16 bytes and value columns to 80 so that the operand reads of
+// a wave fall into different banks).  Long row tiles run first.
+constexpr int kKeyRow = DK + 8;            // elements of a key row in LDS
+constexpr int kValueColumn = 40;           // elements of a value column in LDS (32 keys + padding)
+constexpr int kStage = 32 * kKeyRow + DV * kValueColumn;
+constexpr int kKeyChunks = 32 * (DK / 8), kValueChunks = DV * 4;        // 16-byte chunks of a tile
+constexpr int kKeyLoads = (kKeyChunks + 255) / 256, kValueLoads = (kValueChunks + 255) / 256;
+#ifdef HFEE_KV_SHARED_BLOCKS
+constexpr int SHARED_BLOCKS = HFEE_KV_SHARED_BLOCKS;
+#else
+constexpr int SHARED_BLOCKS = 1;     // (two blocks a wave measured slower: fewer waves to hide the waits)
+#endif
+
+template <int RB>
+__global__ __launch_bounds__(256) void attention_kv_shared_kernel(
+    bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq,
+    const bf16_t* __restrict__ cache, KvLayout lay, const int* __restrict__ items, int num_items,
+    const int* __restrict__ block_tables, int bt_stride, int num_heads, float scale_log2,
+    const float* __restrict__ sinks) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t stages[];
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4, w = threadIdx.x >> 6;
+  const int hpg = num_heads / lay.kv_heads;
+  const int quads = num_heads / 4;
+  const int item = num_items - 1 - (int)(blockIdx.x / quads);
+  const int head = (int)(blockIdx.x % quads) * 4 + w;
+  const int kvh = head / hpg;
+  const int row0 = items[item * 4 + 0], rows = items[item * 4 + 1], pos0 = items[item * 4 + 2];
+  const int* bt = block_tables + (int64_t)items[item * 4 + 3] * bt_stride;
+  const int blocks = (rows + 15) >> 4;
+
+  int token[RB], pos[RB];
+  bool valid[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const int rr = min(16 * b + r, rows - 1);
+    token[b] = row0 + rr; pos[b] = pos0 + rr; valid[b] = 16 * b + r < rows;
+  }
+  Operand qop[RB][KSTEPS];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    const bf16_t* qr = q + (int64_t)token[b] * ldq + (int64_t)head * DK + g * 8;
+#pragma unroll
+    for (int st = 0; st < KSTEPS; ++st) {
+      if (st * 32 + g * 8 < DK) qop[b][st].u = *reinterpret_cast<const u32x4*>(qr + st * 32);
+      else qop[b][st].u = u32x4{0, 0, 0, 0};
+    }
+  }
+  f32x4 acc[RB][VBLOCKS];
+  float m[RB], lsum[RB];
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    m[b] = -INFINITY; lsum[b] = 0.f;
+#pragma unroll
+    for (int vb = 0; vb < VBLOCKS; ++vb) acc[b][vb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int max_pos = pos0 + rows - 1;
+  const int ntiles = (max_pos >> 5) + 1;
+  const int last_block = max_pos >> lay.page_shift;
+  const int slot_mask = lay.page_size - 1;
+
+  // two sets of registers for the chunks on their way, where that is few registers: a tile is then
+  // asked for two tiles before it is multiplied (memory takes longer than one tile's products)
+  constexpr bool DEEP = 4 * (kKeyLoads + kValueLoads) <= 32;
+  u32x4 kst_a[kKeyLoads], vst_a[kValueLoads], kst_b[DEEP ? kKeyLoads : 1], vst_b[DEEP ? kValueLoads : 1];
+  auto fetch = [&](int tile, u32x4* kst, u32x4* vst) {          // this thread's chunks of the tile, into registers
+    const bf16_t* keys[2];
+    const bf16_t* values[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int jb = (tile << 5) + kb * 16;
+      const int page = bt[min(jb >> lay.page_shift, last_block)];
+      keys[kb] = cache + lay.key_offset(page, kvh, jb & slot_mask, 0);
+      values[kb] = cache + lay.values_of(page, kvh) + (jb & slot_mask);
+    }
+#pragma unroll
+    for (int i = 0; i < kKeyLoads; ++i) {
+      const int c = i * 256 + threadIdx.x;
+      if (c < kKeyChunks) {
+        const int row = c / (DK / 8), col = c % (DK / 8);
+        kst[i] = *reinterpret_cast<const u32x4*>(keys[row >> 4] + (row & 15) * DK + col * 8);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kValueLoads; ++i) {
+      const int c = i * 256 + threadIdx.x;
+      if (c < kValueChunks) {
+        const int col = c >> 2, part = c & 3;
+        vst[i] = *reinterpret_cast<const u32x4*>(values[part >> 1] + (int64_t)col * lay.page_size + (part & 1) * 8);
+      }
+    }
+  };
+  auto commit = [&](int buffer, const u32x4* kst, const u32x4* vst) {       // the registers into a stage
+    bf16_t* st = stages + buffer * kStage;
+#pragma unroll
+    for (int i = 0; i < kKeyLoads; ++i) {
+      const int c = i * 256 + threadIdx.x;
+      if (c < kKeyChunks) *reinterpret_cast<u32x4*>(st + (c / (DK / 8)) * kKeyRow + (c % (DK / 8)) * 8) = kst[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kValueLoads; ++i) {
+      const int c = i * 256 + threadIdx.x;
+      if (c < kValueChunks) *reinterpret_cast<u32x4*>(st + 32 * kKeyRow + (c >> 2) * kValueColumn + (c & 3) * 8) = vst[i];
+    }
+  };
+  auto multiply = [&](int tile, const bf16_t* st) {
+    const int j0 = tile << 5;
+    bool live[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) live[b] = b < blocks && j0 <= pos0 + min(rows - 1, 16 * b + 15);
+    f32x4 s[RB][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int b = 0; b < RB; ++b) s[b][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        Operand kop;
+        if (ks * 32 + g * 8 < DK) kop.u = *reinterpret_cast<const u32x4*>(st + (kb * 16 + r) * kKeyRow + ks * 32 + g * 8);
+        else kop.u = u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int b = 0; b < RB; ++b)
+          if (live[b]) s[b][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qop[b][ks].v, s[b][kb], 0, 0, 0);
+      }
+    }
+    Operand pop[RB];
+#pragma unroll
+    for (int b = 0; b < RB; ++b) {
+      if (!live[b]) continue;
+      // (the smallest position of the block's rows: a tile that ends at or before it hides no key)
+      const bool masked = j0 + 31 > pos0 + min(rows - 1, 16 * b);
+      weigh_tile(s[b], m[b], lsum[b], acc[b], pop[b], j0, g, pos[b], scale_log2, masked);
+    }
+#pragma unroll
+    for (int vb = 0; vb < VBLOCKS; ++vb) {
+      Operand vop;
+      const bf16_t* column = st + 32 * kKeyRow + (vb * 16 + r) * kValueColumn + g * 4;
+      vop.h[0] = *reinterpret_cast<const u32x2*>(column);
+      vop.h[1] = *reinterpret_cast<const u32x2*>(column + 16);
+#pragma unroll
+      for (int b = 0; b < RB; ++b) {
+        if (!live[b]) continue;
+        acc[b][vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop.v, pop[b].v, acc[b][vb], 0, 0, 0);
+      }
+    }
+  };
+  fetch(0, kst_a, vst_a);
+  if (DEEP && ntiles > 1) fetch(1, kst_b, vst_b);
+  commit(0, kst_a, vst_a);
+  __syncthreads();
+  if constexpr (DEEP) {
+    for (int tile = 0; tile < ntiles; tile += 2) {
+      if (tile + 2 < ntiles) fetch(tile + 2, kst_a, vst_a);
+      multiply(tile, stages + (tile & 1) * kStage);
+      if (tile + 1 < ntiles) commit((tile + 1) & 1, kst_b, vst_b);
+      __syncthreads();
+      if (tile + 1 >= ntiles) break;
+      if (tile + 3 < ntiles) fetch(tile + 3, kst_b, vst_b);
+      multiply(tile + 1, stages + ((tile + 1) & 1) * kStage);
+      if (tile + 2 < ntiles) commit((tile + 2) & 1, kst_a, vst_a);
+      __syncthreads();
+    }
+  } else {
+    for (int tile = 0; tile < ntiles; ++tile) {
+      if (tile + 1 < ntiles) fetch(tile + 1, kst_a, vst_a);
+      multiply(tile, stages + (tile & 1) * kStage);
+      if (tile + 1 < ntiles) commit((tile + 1) & 1, kst_a, vst_a);
+      __syncthreads();
+    }
+  }
+
+#pragma unroll
+  for (int b = 0; b < RB; ++b) {
+    if (b >= blocks) continue;
+    float l = lsum[b];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    float a = 1.f;
+    if (sinks != nullptr) {
+      const float sk = sinks[head] * kLog2e;
+      const float m_all = fmaxf(m[b], sk);
+      a = exp2f(m[b] - m_all);
+      l = l * a + exp2f(sk - m_all);
+    }
+    if (!valid[b]) continue;
+    const float inv = a / l;
+    bf16_t* orow = out + (int64_t)token[b] * ld_out + (int64_t)head * DV + g * 4;
+#pragma unroll
+    for (int vb = 0; vb < VBLOCKS; ++vb) {
+      const u32x2 wv = {pack_bf16(acc[b][vb][0] * inv, acc[b][vb][1] * inv),
+                        pack_bf16(acc[b][vb][2] * inv, acc[b][vb][3] * inv)};
+      *reinterpret_cast<u32x2*>(orow + vb * 16) = wv;
+    }
+  }
+}
+
 // joins the splits of a single token's heads: one wave per (item, head).  Lane sp holds split sp's
 // maximum and sum (at most 64 splits), the weights of the splits come from one reduction over the
 // wave, and the value dims are then summed over the splits in their order, lanes over the dims.
@@ -252,6 +528,7 @@ __global__ __launch_bounds__(64) void attention_kv_join_kernel(
   const float inv = 1.0f / lsum;
   for (int d = lane; d < DV; d += 64) {
     float o = 0.f;
+#pragma unroll 8
     for (int sp = 0; sp < splits; ++sp) o = fmaf(pr[sp * kPartial + 4 + d], __shfl(my_w, sp, 64), o);
     out[(int64_t)token * ld_out + (int64_t)head * DV + d] = float_to_bf16(o * inv);
   }
@@ -263,8 +540,11 @@ HFEE_DEFINE_LAST_ERROR
 
 HFEE_API int hfee_attention_kv_bf16_dk() { return DK; }
 HFEE_API int hfee_attention_kv_bf16_dv() { return DV; }
-// the most rows of an item of mode 0
-HFEE_API int hfee_attention_kv_bf16_rows() { return 16 * PORTION_BLOCKS; }
+// the most rows of an item of mode 0, for this many query heads a key/value head (where they are a
+// multiple of four, the kernel that shares the key tiles through LDS runs)
+HFEE_API int hfee_attention_kv_bf16_rows(int heads_per_kv_head) {
+  return 16 * (heads_per_kv_head % 4 == 0 ? SHARED_BLOCKS : PORTION_BLOCKS);
+}
 
 // float32 words of `partial` that `splits` > 1 need for `num_items` single tokens
 HFEE_API int64_t hfee_attention_kv_bf16_partial(int num_items, int num_heads, int splits) {
@@ -299,7 +579,21 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
   const int64_t blocks = (waves + 3) / 4;
   HFEE_REQUIRE(blocks <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
   const float scale_log2 = scale * kLog2e;
-  if (mode == 0)
+  if (mode == 0 && hpg % 4 == 0) {
+    const size_t lds = 2 * (size_t)kStage * sizeof(bf16_t);
+    static bool allowed = false;       // (more than 64 KB of LDS has to be asked for once)
+    if (!allowed) {
+      if (hipFuncSetAttribute((const void*)attention_kv_shared_kernel<SHARED_BLOCKS>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return fail("attention_kv_bf16: %zu bytes of LDS are not to be had", lds);
+      allowed = true;
+    }
+    const int64_t groups = (int64_t)num_items * (num_heads / 4);
+    HFEE_REQUIRE(groups <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
+    attention_kv_shared_kernel<SHARED_BLOCKS><<<(unsigned)groups, 256, lds, stream>>>((bf16_t*)out, ld_out,
+        (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads,
+        scale_log2, sinks);
+  } else if (mode == 0)
     attention_kv_kernel<0, PORTION_BLOCKS><<<(unsigned)blocks, 256, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq,
         (const bf16_t*)cache, lay, items, num_items, block_tables, bt_stride, num_heads, scale_log2, sinks, partial, 1);
   else

@@ -38,6 +38,9 @@ ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
 ATTENTION_KV_SOURCE = "attention_kv_bf16.hip"      # compiled per (key size, value size)
 ATTENTION_KV_MOST = (1024, 512)
+# the pairs that `build_all` compiles: those of the tests and of bench.py's comparison (a model with
+# other sizes compiles its own at first use)
+ATTENTION_KV_SIZES = ((32, 16), (48, 32), (16, 48), (112, 96), (64, 64), (128, 96), (128, 128), (576, 512))
 
 
 class BuildError(RuntimeError):
@@ -184,11 +187,12 @@ def build_library(name: str, force: bool = False) -> str:
     return so
 
 
-def build_all(head_dims=HEAD_DIMS, force: bool = True) -> list:
-    """Compiles the core library and the attention library of every head size."""
+def build_all(head_dims=HEAD_DIMS, force: bool = True, kv_sizes=ATTENTION_KV_SIZES) -> list:
+    """Compiles the core library, the attention library of every head size, and the attention
+    libraries for keys and values of different sizes of the listed pairs."""
     out = [build_library("core", force=force)]
     # the attention libraries are independent: build them side by side
-    names = [f"attention_bf16_hd{hd}" for hd in head_dims]
+    names = [f"attention_bf16_hd{hd}" for hd in head_dims] + [f"attention_kv_bf16_k{dk}_v{dv}" for dk, dv in kv_sizes]
     errors = []
 
     def work(n):

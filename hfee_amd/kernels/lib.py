@@ -58,7 +58,7 @@ _CORE_SIGNATURES = {
 _ATTENTION_KV_SIGNATURES = {
     "hfee_attention_kv_bf16_dk": [],
     "hfee_attention_kv_bf16_dv": [],
-    "hfee_attention_kv_bf16_rows": [],
+    "hfee_attention_kv_bf16_rows": [I],
     "hfee_attention_kv_bf16": [P, L, P, L, P, P, I, I, P, I, I, I, I, F, P, P, L, I, P],
 }
 

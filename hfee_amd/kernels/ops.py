@@ -873,9 +873,10 @@ def attention_kv_sizes_fit(dk: int, dv: int) -> bool:
     return dk % 16 == 0 and dv % 16 == 0 and 16 <= dk <= build.ATTENTION_KV_MOST[0] and 16 <= dv <= build.ATTENTION_KV_MOST[1]
 
 
-def attention_kv_rows(dk: int, dv: int) -> int:
-    """The most rows that an item of `attention_kv_bf16`'s mode 0 may hold for these sizes."""
-    return int(lib.attention_kv_bf16(dk, dv).raw("hfee_attention_kv_bf16_rows")())
+def attention_kv_rows(dk: int, dv: int, heads_per_kv_head: int = 1) -> int:
+    """The most rows that an item of `attention_kv_bf16`'s mode 0 may hold for these sizes and this
+    many query heads a key/value head."""
+    return int(lib.attention_kv_bf16(dk, dv).raw("hfee_attention_kv_bf16_rows")(int(heads_per_kv_head)))
 
 
 def attention_kv_partial_words(num_items: int, num_heads: int, dv: int, splits: int) -> int:

@@ -62,7 +62,7 @@ def attend(ctx, out, q, cache, tables, num_heads, kv_heads, dk, dv, scale, sinks
         ops.attention_kv_plain(out, q, cache, ctx.positions, ctx.token_segment, tables, num_heads, kv_heads, dk, dv,
                                ctx.page_size, scale, sinks)
         return
-    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv)}"]
+    portions = ctx.extra[f"attention_kv.portions.{ops.attention_kv_rows(dk, dv, num_heads // kv_heads)}"]
     singles = ctx.extra["attention_kv.singles"]
     if portions.shape[0]:
         ops.attention_kv_bf16(out, q, cache, portions, 0, tables, num_heads, kv_heads, dk, dv, ctx.page_size, scale, sinks)
@@ -150,7 +150,7 @@ class KvAttention(_KvMixer):
                                             sink="sinks", value_blend="value_blend"))
         self.q_width, self.k_width, self.v_width = self.num_heads * self.dk, self.kv_heads * self.dk, self.kv_heads * self.dv
         self.out_width = self.num_heads * self.dv
-        self.kernel_sizes = (self.dk, self.dv)
+        self.kernel_sizes = (self.dk, self.dv, self.num_heads // self.kv_heads)
         self.matrix = self._matrix(self.dk, self.dv, self.q_width + self.k_width + self.v_width, self.out_width)
 
     def tensor_specs(self):
@@ -227,7 +227,7 @@ class LatentAttention(_KvMixer):
                                             v_up="v_b_proj.weight", o="o_proj.weight"))
         # the absorbed form: one key/value head, keys [latent | rotated part], values the latent
         self.dk_abs, self.dv_abs = self.kv_rank + self.rotated, self.kv_rank
-        self.kernel_sizes = (self.dk_abs, self.dv_abs)
+        self.kernel_sizes = (self.dk_abs, self.dv_abs, self.num_heads)
         self.down_width = self.q_rank + self.kv_rank + self.rotated
         self.matrix = (self._matrix(self.dk_abs, self.dv_abs, self.num_heads * self.dk_abs, self.num_heads * self.dv_abs)
                        and self.down_width % 8 == 0 and self.q_rank % 8 == 0)

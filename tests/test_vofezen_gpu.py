@@ -135,7 +135,7 @@ def test_attention_kernels(dtype, H, G, dk, dv):
     assert vu.rel(out.double().cpu(), no_sink) < tol
     if dtype == "float32" or not ops.attention_kv_sizes_fit(dk, dv):
         return
-    items0, row, most = [], 0, ops.attention_kv_rows(dk, dv)
+    items0, row, most = [], 0, ops.attention_kv_rows(dk, dv, H // G)
     for s, (st, ln) in enumerate(zip(starts, lengths)):
         if ln > 1:
             items0 += [(row + off, min(most, ln - off), st + off, s) for off in range(0, ln, most)]
