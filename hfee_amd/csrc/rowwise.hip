@@ -130,6 +130,26 @@ __global__ void bias_act_kernel(T* __restrict__ out, int64_t ldo, const T* __res
   out[row * ldo + j] = from_float<T>(activate(z, act));
 }
 
+// eight bfloat16 values a thread (16 bytes), for widths that are multiples of 8 and aligned rows
+__global__ void bias_act_bf16x8_kernel(bf16_t* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ in, int64_t ldi,
+                                       const bf16_t* __restrict__ bias, int width, int act) {
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  const int64_t row = blockIdx.y;
+  const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (j >= width) return;
+  const u32x4_t v = *reinterpret_cast<const u32x4_t*>(in + row * ldi + j);
+  u32x4_t b = {0, 0, 0, 0};
+  if (bias != nullptr) b = *reinterpret_cast<const u32x4_t*>(bias + j);
+  u32x4_t o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float lo = activate(bf16_to_float((bf16_t)(v[i] & 0xffff)) + bf16_to_float((bf16_t)(b[i] & 0xffff)), act);
+    const float hi = activate(bf16_to_float((bf16_t)(v[i] >> 16)) + bf16_to_float((bf16_t)(b[i] >> 16)), act);
+    o[i] = (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
+  }
+  *reinterpret_cast<u32x4_t*>(out + row * ldo + j) = o;
+}
+
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void rmsnorm_cols_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ x,
                                                            int64_t ldx, const TW* __restrict__ w, float offset,
@@ -214,10 +234,15 @@ HFEE_API int hfee_bias_act(void* out, int64_t ldo, const void* in, int64_t ldi, 
   HFEE_REQUIRE(act >= ACT_NONE && act <= ACT_SILU, "bias_act: unknown activation %d", act);
   HFEE_REQUIRE(n <= 65535 * 32, "bias_act: too many rows");
   if (n == 0) return 0;
+  const bool wide = dtype == 1 && width % 8 == 0 && ldo % 8 == 0 && ldi % 8 == 0 &&
+                    ((uintptr_t)out | (uintptr_t)in | (uintptr_t)bias) % 16 == 0;
   for (int r0 = 0; r0 < n; r0 += 65535) {
     const int rows = n - r0 < 65535 ? n - r0 : 65535;
     dim3 grid((width + 255) / 256, rows);
-    if (dtype == 0)
+    if (wide)
+      bias_act_bf16x8_kernel<<<dim3((width / 8 + 255) / 256, rows), 256, 0, stream>>>(
+          (bf16_t*)out + (int64_t)r0 * ldo, ldo, (const bf16_t*)in + (int64_t)r0 * ldi, ldi, (const bf16_t*)bias, width, act);
+    else if (dtype == 0)
       bias_act_kernel<float><<<grid, 256, 0, stream>>>((float*)out + (int64_t)r0 * ldo, ldo, (const float*)in + (int64_t)r0 * ldi,
                                                         ldi, (const float*)bias, width, act);
     else if (dtype == 1)

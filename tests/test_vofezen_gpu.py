@@ -89,7 +89,7 @@ def softmax_rows(q, k, v, scale, positions, sink=None):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H,G,dk,dv", [(4, 2, 32, 16), (20, 1, 16, 48), (3, 3, 24, 28), (6, 1, 128, 96), (5, 5, 64, 64)])
+@pytest.mark.parametrize("H,G,dk,dv", [(4, 2, 32, 16), (20, 1, 16, 48), (3, 3, 24, 28), (8, 1, 160, 128), (5, 5, 64, 64)])
 def test_attention_kernels(dtype, H, G, dk, dv):
     """Plain and matrix-core kernels, portions and single tokens (keys split and not), a sink, stale
     numbers in the pages, one far key that outweighs hundreds, and a sink that outweighs all keys."""
@@ -219,6 +219,9 @@ def test_row_kernels(dtype):
         out = torch.zeros((n, d), dtype=dt, device="cuda")
         ops.bias_act(out, dev(z, dt), dev(zb, dt), act)
         assert vu.rel(out.double().cpu(), f(z + zb)) < tol, act
+        out = torch.zeros((n, 48), dtype=dt, device="cuda")          # (a width that takes eight values a thread)
+        ops.bias_act(out, dev(z[:, :48], dt), dev(zb[:48], dt), act)
+        assert vu.rel(out.double().cpu(), f(z[:, :48] + zb[:48])) < tol, act
     wide = dev(z, dt)
     cols = wide[:, 7:47]
     w = 1 + rng.standard_normal(40) * 0.2
