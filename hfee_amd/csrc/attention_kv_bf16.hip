@@ -322,6 +322,8 @@ constexpr int kValueColumn = 40;           // elements of a value column in LDS 
 constexpr int kStage = 32 * kKeyRow + DV * kValueColumn;
 constexpr int kKeyChunks = 32 * (DK / 8), kValueChunks = DV * 4;        // 16-byte chunks of a tile
 constexpr int kKeyLoads = (kKeyChunks + 255) / 256, kValueLoads = (kValueChunks + 255) / 256;
+// (two stages have to fit the 160 KB of a CU; sizes beyond that take the kernel without LDS)
+constexpr bool kSharedFits = 2 * (size_t)kStage * sizeof(bf16_t) <= 160 * 1024;
 #ifdef HFEE_KV_SHARED_BLOCKS
 constexpr int SHARED_BLOCKS = HFEE_KV_SHARED_BLOCKS;
 #else
@@ -543,7 +545,7 @@ HFEE_API int hfee_attention_kv_bf16_dv() { return DV; }
 // the most rows of an item of mode 0, for this many query heads a key/value head (where they are a
 // multiple of four, the kernel that shares the key tiles through LDS runs)
 HFEE_API int hfee_attention_kv_bf16_rows(int heads_per_kv_head) {
-  return 16 * (heads_per_kv_head % 4 == 0 ? SHARED_BLOCKS : PORTION_BLOCKS);
+  return 16 * (kSharedFits && heads_per_kv_head % 4 == 0 ? SHARED_BLOCKS : PORTION_BLOCKS);
 }
 
 // float32 words of `partial` that `splits` > 1 need for `num_items` single tokens
@@ -579,7 +581,7 @@ HFEE_API int hfee_attention_kv_bf16(void* out, int64_t ld_out, const void* q, in
   const int64_t blocks = (waves + 3) / 4;
   HFEE_REQUIRE(blocks <= 0x7fffffff, "attention_kv_bf16: too much work for one launch");
   const float scale_log2 = scale * kLog2e;
-  if (mode == 0 && hpg % 4 == 0) {
+  if (mode == 0 && kSharedFits && hpg % 4 == 0) {
     const size_t lds = 2 * (size_t)kStage * sizeof(bf16_t);
     static bool allowed = false;       // (more than 64 KB of LDS has to be asked for once)
     if (!allowed) {

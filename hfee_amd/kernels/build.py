@@ -40,7 +40,7 @@ ATTENTION_KV_SOURCE = "attention_kv_bf16.hip"      # compiled per (key size, val
 ATTENTION_KV_MOST = (1024, 512)
 # the pairs that `build_all` compiles: those of the tests and of bench.py's comparison (a model with
 # other sizes compiles its own at first use)
-ATTENTION_KV_SIZES = ((32, 16), (48, 32), (16, 48), (112, 96), (64, 64), (160, 128), (128, 128), (576, 512))
+ATTENTION_KV_SIZES = ((32, 16), (64, 32), (96, 64), (48, 32), (16, 48), (112, 96), (64, 64), (160, 128), (128, 128), (576, 512))
 
 
 class BuildError(RuntimeError):

@@ -22,7 +22,8 @@ pytestmark = pytest.mark.gpu
 
 TOL = {"float32": 3e-5, "bfloat16": 5e-2}
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
-LENGTHS = {"A": [5, 17, 64, 1, 100, 33, 129, 49, 2], "B": [40, 3, 100, 65, 2, 31], "C": [150, 70, 700, 41, 97]}
+LENGTHS = {"A": [5, 17, 64, 1, 100, 33, 129, 49, 2], "B": [40, 3, 100, 65, 2, 31], "C": [150, 70, 700, 41, 97],
+           "D": [1300, 47, 513, 1]}
 
 
 def dev(a, dtype=None):
@@ -281,7 +282,7 @@ def compare(got, want, tol, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_every_way_of_cutting_gives_the_plain_logits(folders, plain_rows, name, dtype):
     from hfee_amd.trace_replay import Replayer
     reqs, want = plain_rows(name, dtype)

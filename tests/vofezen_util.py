@@ -55,7 +55,16 @@ V_C = config(300, 128, 1e-5, [
     with_mlp(latent(1, 32, 16, 48, 64, 96), 256),
     with_mlp(attention(20, 1, 16, 48, 8, True), 64),
 ])
-CONFIGS = {"A": V_A, "B": V_B, "C": V_C}
+# latent attention first, four query heads a key/value head and eight latent heads (the kernels that
+# share key tiles through LDS), larger sizes, for prompts beyond a thousand tokens
+V_D = config(1000, 256, 1e-6, [
+    with_mlp(latent(8, 32, 32, 48, 96, 64), 384),
+    with_mlp(attention(8, 2, 64, 32, 32, True, base=50000.0), 320),
+    with_mlp(attention(8, 2, 64, 32, 32, False, base=50000.0), None),
+    with_mlp(attention(8, 2, 64, 32, 32, True, base=50000.0), 384),
+    with_mlp(latent(8, 32, 32, 48, 96, 64), 128),
+])
+CONFIGS = {"A": V_A, "B": V_B, "C": V_C, "D": V_D}
 
 
 def make_folder(path, config_json, seed, dtype="float32", std=0.1):
