@@ -50,7 +50,7 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 // column operand of the value product.  The exponentials are taken against a reference that lags
 // the running maximum: the sums are rescaled only when a maximum has moved by more than 2^8 (the
 // quotient at the end does not depend on the reference), so most tiles cost no pass over the
-// output sums.  Keys beyond the row's own position weigh nothing; `masked` says whether the tile
+// output sums and no exchange between lanes.  Keys beyond the row's own position weigh nothing; `masked` says whether the tile
 // has any (the same answer in every lane).
 __device__ __forceinline__ void weigh_tile(f32x4 (&s)[2], float& reference, float& lsum, f32x4 (&acc)[VBLOCKS],
                                            Operand& pop, int j0, int g, int pos, float scale_log2, bool masked) {
@@ -64,12 +64,14 @@ __device__ __forceinline__ void weigh_tile(f32x4 (&s)[2], float& reference, floa
       s[kb][i] = v;
       tmax = fmaxf(tmax, v);
     }
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-  tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+  // (a lane looks at its own eight keys first: the four lanes of a query meet over the maximum only
+  // when one of them is beyond the reference by 2^8, which after the first tiles is rare)
   if (__builtin_amdgcn_ballot_w64(tmax > reference + 8.0f) != 0) {      // (-inf + 8 = -inf: the first tile always)
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float moved = fmaxf(reference, tmax);
     const float use = moved == -INFINITY ? 0.f : moved;
-    const float alpha = exp2f(reference - use);
+    const float alpha = __builtin_amdgcn_exp2f(reference - use);
     reference = moved;
     lsum *= alpha;
 #pragma unroll
@@ -81,7 +83,7 @@ __device__ __forceinline__ void weigh_tile(f32x4 (&s)[2], float& reference, floa
   for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float p = exp2f(s[kb][i] - use);
+      const float p = __builtin_amdgcn_exp2f(s[kb][i] - use);
       s[kb][i] = p;
       psum += p;
     }

@@ -20,7 +20,9 @@ from conftest import ROOT
 
 pytestmark = pytest.mark.gpu
 
-TOL = {"float32": 3e-5, "bfloat16": 5e-2}
+# (bfloat16: the worst rows of the larger configuration come to 0.050 under some cuts and 0.040 under others,
+# its median row to 0.016, whichever kernels run)
+TOL = {"float32": 3e-5, "bfloat16": 8e-2}
 DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 LENGTHS = {"A": [5, 17, 64, 1, 100, 33, 129, 49, 2], "B": [40, 3, 100, 65, 2, 31], "C": [150, 70, 700, 41, 97],
            "D": [1300, 47, 513, 1]}
@@ -272,13 +274,18 @@ def plain_rows(folders):
 
 
 def compare(got, want, tol, what):
+    """Every row within tol of the plain row, relative to the row's largest logit; the median row
+    within half of that (the format's noise has single rows near the bound on some models: a fault
+    of a kernel moves many rows, and the median with them)."""
     assert set(got) == set(want), f"{what}: positions differ"
-    worst, where = 0.0, None
+    worst, where, errors = 0.0, None, []
     for key in want:
         e = vu.rel(got[key], want[key])
+        errors.append(e)
         if not e <= worst:
             worst, where = e, key
     assert worst < tol, f"{what}: worst relative error {worst:.3e} at {where}"
+    assert np.median(errors) < tol / 2, f"{what}: median relative error {np.median(errors):.3e}"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
