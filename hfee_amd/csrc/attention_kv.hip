@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
 // Lane (j mod 64) owns key j, so which lane adds which term depends only on the key's
 // absolute position: a token's result does not change with the way the work was cut into
 // steps, with the batch around it or with page numbers.
-constexpr int kMaxDvPerLane = 8;      // value sizes up to 512
+constexpr int kMaxDvPerLane = 16;     // value sizes up to 1,024
 
 template <typename T>
 __global__ __launch_bounds__(64) void attention_kv_plain_kernel(
