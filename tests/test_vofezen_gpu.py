@@ -373,3 +373,31 @@ def test_trace_runner_as_a_subprocess(folders, tmp_path):
     assert not (out / "1.f32").exists()
     assert vu.rel(a[0], want[0]) < 3e-5 and vu.rel(a[1], want[20]) < 3e-5
     assert vu.rel(c[0], want[38]) < 3e-5 and vu.rel(c[1], want[1]) < 3e-5
+
+
+def test_the_command_line_runs_the_design(folders):
+    """`hfee run <folder> --tokens ...`: the greedy continuation's ids."""
+    folder = folders[("B", "float32")]
+    prompt = tu.make_requests(97, [11], seed=8)["r0"]
+    want = pv.PlainVofezen(folder).greedy(prompt, 7)
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "hfee"), "run", folder, "--tokens",
+                        ",".join(map(str, prompt)), "--dtype", "float32", "--temperature", "0", "--repeat-penalty", "1",
+                        "--num-predict", "7", "--num-ctx", "128", "--verbose"],
+                       capture_output=True, text=True, timeout=300, stdin=subprocess.DEVNULL)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [int(t) for t in p.stdout.strip().splitlines()[0].split()] == want
+    assert "prompt eval count:    11 token(s)" in p.stdout and "eval count:           7 token(s)" in p.stdout
+
+
+def test_seeded_sampling_does_not_depend_on_the_batch(folders):
+    """The sampler's contract holds for this design too: a request's seeded draws are the same
+    alone and beside others."""
+    from hfee_amd import LLM, SamplingParams
+    folder = folders[("A", "float32")]
+    g = np.random.default_rng(3)
+    prompts = [g.integers(0, 211, size=n).tolist() for n in (9, 30, 2)]
+    params = [SamplingParams(temperature=0.9, top_k=20, top_p=0.95, seed=100 + i, num_predict=10) for i in range(3)]
+    together = LLM(folder, dtype="float32", num_ctx=128, num_parallel=3).generate(prompts, params)
+    for i in range(3):
+        alone = LLM(folder, dtype="float32", num_ctx=128, num_parallel=1).generate([prompts[i]], [params[i]])[0]
+        assert alone.token_ids == together[i].token_ids
