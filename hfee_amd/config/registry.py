@@ -57,8 +57,20 @@ def config_from_dict(config_json: dict, where: str = "config.json"):
 
 
 def config_from_folder(model_dir: str):
+    """A configuration class with `reads_tensor_shapes = True` also gets the shapes of the folder's
+    tensors (from the checkpoint's header; no data is read): sizes that config.json leaves to them."""
     data = read_config_json(model_dir)
-    return config_from_dict(data, where=f"{model_dir}/config.json")
+    where = f"{model_dir}/config.json"
+    arch = architecture_of(data, where)
+    if getattr(arch.config_class, "reads_tensor_shapes", False):
+        from ..weights.safetensors_io import Checkpoint, SafetensorsError
+        try:
+            ckpt = Checkpoint(model_dir)
+            shapes = {n: tuple(ckpt.entry(n).shape) for n in ckpt.names()}
+        except (SafetensorsError, OSError):
+            shapes = None          # (a folder with a configuration only: random weights)
+        return arch.config_class.from_dict(data, where, tensor_shapes=shapes)
+    return arch.config_class.from_dict(data, where)
 
 
 def model_spec_of(config) -> ModelSpec:

@@ -20,17 +20,17 @@ HFEE_DEFINE_LAST_ERROR
 // ------------------------------------------------------------------ embedding
 template <typename T>
 __global__ void embed_kernel(float* __restrict__ out, const T* __restrict__ table,
-                             const int* __restrict__ ids, int d) {
+                             const int* __restrict__ ids, int d, float scale) {
   const int row = blockIdx.x;
   const int64_t src = (int64_t)ids[row] * d;
-  for (int j = threadIdx.x; j < d; j += blockDim.x) out[(int64_t)row * d + j] = to_float<T>(table[src + j]);
+  for (int j = threadIdx.x; j < d; j += blockDim.x) out[(int64_t)row * d + j] = to_float<T>(table[src + j]) * scale;
 }
 
 // bfloat16 rows of a width that is a multiple of 8, 16-byte aligned: eight elements a
 // thread, a row over several workgroups (a decode step's few rows then take one round of
 // loads, not sixteen one after the other)
 __global__ __launch_bounds__(256) void embed_bf16_wide_kernel(float* __restrict__ out, const bf16_t* __restrict__ table,
-                                                              const int* __restrict__ ids, int d) {
+                                                              const int* __restrict__ ids, int d, float scale) {
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   const int row = blockIdx.x, j = 8 * (blockIdx.y * 256 + threadIdx.x);
@@ -45,8 +45,8 @@ __global__ __launch_bounds__(256) void embed_bf16_wide_kernel(float* __restrict_
     hi[2 * i] = __uint_as_float(v[2 + i] << 16);
     hi[2 * i + 1] = __uint_as_float(v[2 + i] & 0xffff0000u);
   }
-  *reinterpret_cast<f32x4*>(o) = lo;
-  *reinterpret_cast<f32x4*>(o + 4) = hi;
+  *reinterpret_cast<f32x4*>(o) = lo * scale;
+  *reinterpret_cast<f32x4*>(o + 4) = hi * scale;
 }
 
 // The same for at most 64 rows, with the first half of the norm that follows: also
@@ -115,19 +115,20 @@ HFEE_API int hfee_embed_emit(float* out, const void* table, const int* ids, int 
   return 0;
 }
 
+// scale: what every element is multiplied by on its way into the stream (1 for a plain lookup).
 HFEE_API int hfee_embed(float* out, const void* table, int table_dtype, const int* ids,
-                        int n, int d, hipStream_t stream) {
+                        int n, int d, float scale, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && d > 0, "embed: bad sizes n=%d d=%d", n, d);
   if (n == 0) return 0;
   if (table_dtype == DT_BF16 && d % 8 == 0 && (uintptr_t)table % 16 == 0 && (uintptr_t)out % 16 == 0 && n <= 65535) {
-    embed_bf16_wide_kernel<<<dim3(n, (d + 2047) / 2048), 256, 0, stream>>>(out, (const bf16_t*)table, ids, d);
+    embed_bf16_wide_kernel<<<dim3(n, (d + 2047) / 2048), 256, 0, stream>>>(out, (const bf16_t*)table, ids, d, scale);
     HFEE_CHECK_LAUNCH("embed");
     return 0;
   }
   if (table_dtype == DT_F32)
-    embed_kernel<float><<<n, 256, 0, stream>>>(out, (const float*)table, ids, d);
+    embed_kernel<float><<<n, 256, 0, stream>>>(out, (const float*)table, ids, d, scale);
   else if (table_dtype == DT_BF16)
-    embed_kernel<bf16_t><<<n, 256, 0, stream>>>(out, (const bf16_t*)table, ids, d);
+    embed_kernel<bf16_t><<<n, 256, 0, stream>>>(out, (const bf16_t*)table, ids, d, scale);
   else
     return fail("embed: unknown dtype %d", table_dtype);
   HFEE_CHECK_LAUNCH("embed");

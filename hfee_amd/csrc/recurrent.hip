@@ -1,0 +1,300 @@
+// Mixers that carry a matrix of fixed size from token to token instead of a growing cache.
+//
+// A head keeps S [D][V] in float32 for every request slot.  With a decay a_t [D] (one number a key
+// channel, acting on the rows of S), a key k_t [D], a value v_t [V] and a query q_t [D]:
+//
+//   rule 0 (gated linear attention):  S <- diag(a_t) S + k_t v_t^T;                    o_t = S^T q_t
+//   rule 1 (gated delta rule):        S <- diag(a_t) S;  u = b_t (v_t - S^T k_t);
+//                                     S <- S + k_t u^T;                                o_t = S^T q_t
+//
+// `linear_scan` walks the tokens that a step brings for a request one after the other, from the
+// state that the steps before left in the request's slot, and leaves the new state there: a
+// portion of a prompt and a single token are the same kernel, and a token's result does not
+// depend on where its prompt was cut.  A thread owns D/4 rows of one column of S; four lanes
+// share a column and add their parts up in a fixed order.
+//
+// Around it, each in float32 whatever the engine's dtype:
+//   short_conv_silu     y_t = silu(sum_j taps[K-1-j] x_(t-j)) per channel, the K-1 inputs before the
+//                       step's first token from the slot's state (zeros at a sequence's start)
+//   short_conv_keep     the slot's state <- the last K-1 inputs
+//   unit_heads          x / sqrt(sum(x^2) + eps) * factor over each head
+//   scan_gate           what a projection becomes before it enters the recurrence:
+//                       0  exp(-exp(A[head]) softplus(z + bias))      (a decay from a step size)
+//                       1  exp(logsigmoid(z + bias) / tau)            (a decay sigmoid(z)^(1/tau))
+//                       2  sigmoid(z)                                 (a writing strength)
+//                       3  z * factor for the first columns, z for the rest (a cast)
+//   head_norm_gate      out = o / sqrt(mean(o^2) + eps) * weight * act(gate) over each head,
+//                       act the sigmoid or the SiLU, in the engine's dtype for the product behind it
+#include "common.h"
+
+using namespace hfee;
+
+namespace {
+
+__device__ __forceinline__ float softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+// x: [n, C] rows of the step; state: [slots][K-1][C], index K-2 the newest; taps: float32 [C][K], the
+// last column the current token's; y: float32 [n, C].
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_silu_kernel(
+    float* __restrict__ y, int64_t ldy, const T* __restrict__ x, int64_t ldx, const T* __restrict__ state,
+    const float* __restrict__ taps, const int* __restrict__ token_segment, const int* __restrict__ segment_rows,
+    const int* __restrict__ segment_slots, int C, int K) {
+  const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int seg = token_segment[t];
+  const int i = t - segment_rows[seg];                      // the token's place in its portion
+  const T* st = state + (int64_t)segment_slots[seg] * (K - 1) * C;
+  float sum = 0.f;
+  for (int j = K - 1; j >= 0; --j) {                        // the oldest input first
+    const int at = i - j;
+    const float v = at >= 0 ? to_float<T>(x[(int64_t)(t - j) * ldx + c]) : to_float<T>(st[(int64_t)(K - 1 + at) * C + c]);
+    sum = fmaf(taps[(int64_t)c * K + (K - 1 - j)], v, sum);
+  }
+  y[(int64_t)t * ldy + c] = sum / (1.0f + expf(-sum));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_keep_kernel(
+    T* __restrict__ state, const T* __restrict__ x, int64_t ldx, const int* __restrict__ segment_rows,
+    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int C, int K) {
+  const int seg = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int len = segment_lengths[seg], row0 = segment_rows[seg];
+  T* st = state + (int64_t)segment_slots[seg] * (K - 1) * C;
+  for (int m = 0; m < K - 1; ++m) {                         // ascending: what is read lies behind what was written
+    const int i = len - (K - 1) + m;
+    st[(int64_t)m * C + c] = i >= 0 ? x[(int64_t)(row0 + i) * ldx + c] : st[(int64_t)(m + len) * C + c];
+  }
+}
+
+// One wave a (token, head): x float32 [n, heads * D], in place.
+__global__ __launch_bounds__(256) void unit_heads_kernel(float* __restrict__ x, int64_t ldx, int heads, int D, float eps,
+                                                         float factor, int n) {
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= (int64_t)n * heads) return;
+  const int lane = threadIdx.x & 63;
+  float* p = x + item / heads * ldx + item % heads * D;
+  float ss = 0.f;
+  for (int d = lane; d < D; d += 64) ss = fmaf(p[d], p[d], ss);
+  const float inv = factor / sqrtf(wave_sum(ss) + eps);
+  for (int d = lane; d < D; d += 64) p[d] *= inv;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void scan_gate_kernel(float* __restrict__ out, int64_t ldo, const T* __restrict__ z,
+                                                        int64_t ldz, const float* __restrict__ bias,
+                                                        const float* __restrict__ per_head, int head_width, int mode,
+                                                        float number, int first_columns, int width) {
+  const int64_t t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  float v = to_float<T>(z[t * ldz + c]);
+  if (bias != nullptr) v += bias[c];
+  float r;
+  if (mode == 0) r = expf(-expf(per_head[c / head_width]) * softplus(v));
+  else if (mode == 1) r = expf(log_sigmoid(v) / number);
+  else if (mode == 2) r = 1.0f / (1.0f + expf(-v));
+  else r = c < first_columns ? v * number : v;
+  out[t * ldo + c] = r;
+}
+
+// grid (column blocks of 16, heads, segments), 64 threads: lane = 16 (part of D) + column.
+template <int DPT, int RULE>
+__global__ __launch_bounds__(64) void linear_scan_kernel(
+    float* __restrict__ out, int64_t ldo, float* __restrict__ state, const float* __restrict__ q, int64_t ldq,
+    const float* __restrict__ k, int64_t ldk, const float* __restrict__ v, int64_t ldv, const float* __restrict__ decay,
+    int64_t ldd, const float* __restrict__ beta, int64_t ldb, const int* __restrict__ segment_rows,
+    const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int heads, int qk_heads, int D, int V) {
+  const int seg = blockIdx.z, h = blockIdx.y;
+  const int col = blockIdx.x * 16 + (threadIdx.x & 15), part = threadIdx.x >> 4;
+  const bool live = col < V;
+  const int d0 = part * DPT;
+  const int g = h / (heads / qk_heads);
+  float* S = state + (((int64_t)segment_slots[seg] * heads + h) * D) * V + (live ? col : 0);
+  float s[DPT];
+#pragma unroll
+  for (int i = 0; i < DPT; ++i) s[i] = live && d0 + i < D ? S[(int64_t)(d0 + i) * V] : 0.f;
+  const int row0 = segment_rows[seg], len = segment_lengths[seg];
+  for (int t = row0; t < row0 + len; ++t) {
+    const float* qt = q + (int64_t)t * ldq + (int64_t)g * D + d0;
+    const float* kt = k + (int64_t)t * ldk + (int64_t)g * D + d0;
+    const float* at = decay + (int64_t)t * ldd + (int64_t)h * D + d0;
+    float kk[DPT], qq[DPT], aa[DPT];
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      const bool in = d0 + i < D;
+      kk[i] = in ? kt[i] : 0.f;
+      qq[i] = in ? qt[i] : 0.f;
+      aa[i] = in ? at[i] : 0.f;
+    }
+    const float vt = live ? v[(int64_t)t * ldv + (int64_t)h * V + col] : 0.f;
+    float u = vt;
+    if constexpr (RULE == 1) {
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) {
+        s[i] *= aa[i];
+        dot = fmaf(s[i], kk[i], dot);
+      }
+      dot += __shfl_xor(dot, 16, kWave);
+      dot += __shfl_xor(dot, 32, kWave);
+      u = beta[(int64_t)t * ldb + h] * (vt - dot);
+    }
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      if constexpr (RULE == 1) s[i] = fmaf(kk[i], u, s[i]);
+      else s[i] = fmaf(s[i], aa[i], kk[i] * u);
+      o = fmaf(s[i], qq[i], o);
+    }
+    o += __shfl_xor(o, 16, kWave);
+    o += __shfl_xor(o, 32, kWave);
+    if (live && part == 0) out[(int64_t)t * ldo + (int64_t)h * V + col] = o;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < DPT; ++i)
+      if (d0 + i < D) S[(int64_t)(d0 + i) * V] = s[i];
+  }
+}
+
+// One wave a (token, head).  o: float32 [n, heads * V]; gate: [n, heads * V] in T; weight: float32 [V].
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(T* __restrict__ out, int64_t ldo, const float* __restrict__ o,
+                                                             int64_t ldi, const T* __restrict__ gate, int64_t ldg,
+                                                             const float* __restrict__ weight, int heads, int V,
+                                                             float eps, int act, int n) {
+  const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (item >= (int64_t)n * heads) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = item / heads, h = item % heads;
+  const float* p = o + t * ldi + h * V;
+  float ss = 0.f;
+  for (int d = lane; d < V; d += 64) ss = fmaf(p[d], p[d], ss);
+  const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
+  for (int d = lane; d < V; d += 64) {
+    const float z = to_float<T>(gate[t * ldg + h * V + d]);
+    const float sig = 1.0f / (1.0f + expf(-z));
+    out[t * ldo + h * V + d] = from_float<T>(p[d] * inv * weight[d] * (act == 0 ? sig : z * sig));
+  }
+}
+
+}  // namespace
+
+HFEE_API int hfee_short_conv_silu(float* y, int64_t ldy, const void* x, int64_t ldx, const void* state, int dtype,
+                                  const float* taps, const int* token_segment, const int* segment_rows,
+                                  const int* segment_slots, int channels, int taps_count, int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && channels > 0 && taps_count >= 1 && taps_count <= 64, "short_conv_silu: bad sizes");
+  if (n == 0) return 0;
+  HFEE_REQUIRE(ldx >= channels && ldy >= channels && (channels + 255) / 256 <= 65535, "short_conv_silu: rows too short or too wide");
+  dim3 grid(n, (channels + 255) / 256);
+  if (dtype == 0)
+    short_conv_silu_kernel<float><<<grid, 256, 0, stream>>>(y, ldy, (const float*)x, ldx, (const float*)state, taps,
+        token_segment, segment_rows, segment_slots, channels, taps_count);
+  else if (dtype == 1)
+    short_conv_silu_kernel<bf16_t><<<grid, 256, 0, stream>>>(y, ldy, (const bf16_t*)x, ldx, (const bf16_t*)state, taps,
+        token_segment, segment_rows, segment_slots, channels, taps_count);
+  else
+    return fail("short_conv_silu: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("short_conv_silu");
+  return 0;
+}
+
+HFEE_API int hfee_short_conv_keep(void* state, const void* x, int64_t ldx, int dtype, const int* segment_rows,
+                                  const int* segment_lengths, const int* segment_slots, int channels, int taps_count,
+                                  int segments, hipStream_t stream) {
+  HFEE_REQUIRE(segments >= 0 && segments <= 65535 && channels > 0 && taps_count >= 1, "short_conv_keep: bad sizes");
+  if (segments == 0 || taps_count == 1) return 0;
+  dim3 grid((channels + 255) / 256, segments);
+  if (dtype == 0)
+    short_conv_keep_kernel<float><<<grid, 256, 0, stream>>>((float*)state, (const float*)x, ldx, segment_rows,
+        segment_lengths, segment_slots, channels, taps_count);
+  else if (dtype == 1)
+    short_conv_keep_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)state, (const bf16_t*)x, ldx, segment_rows,
+        segment_lengths, segment_slots, channels, taps_count);
+  else
+    return fail("short_conv_keep: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("short_conv_keep");
+  return 0;
+}
+
+HFEE_API int hfee_unit_heads(float* x, int64_t ldx, int heads, int dim, float eps, float factor, int n, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && heads > 0 && dim > 0 && ldx >= (int64_t)heads * dim, "unit_heads: bad sizes");
+  if (n == 0) return 0;
+  const int64_t items = (int64_t)n * heads;
+  unit_heads_kernel<<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(x, ldx, heads, dim, eps, factor, n);
+  HFEE_CHECK_LAUNCH("unit_heads");
+  return 0;
+}
+
+HFEE_API int hfee_scan_gate(float* out, int64_t ldo, const void* z, int64_t ldz, int dtype, const float* bias,
+                            const float* per_head, int head_width, int mode, float number, int first_columns, int n,
+                            int width, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && width > 0 && (width + 255) / 256 <= 65535 && ldo >= width && ldz >= width, "scan_gate: bad sizes");
+  HFEE_REQUIRE(mode >= 0 && mode <= 3, "scan_gate: unknown mode %d", mode);
+  HFEE_REQUIRE(mode != 0 || (per_head != nullptr && head_width > 0), "scan_gate: a decay from a step size needs a number a head");
+  HFEE_REQUIRE(mode != 1 || number > 0.f, "scan_gate: tau must be positive");
+  if (n == 0) return 0;
+  dim3 grid(n, (width + 255) / 256);
+  if (dtype == 0)
+    scan_gate_kernel<float><<<grid, 256, 0, stream>>>(out, ldo, (const float*)z, ldz, bias, per_head, head_width, mode,
+                                                      number, first_columns, width);
+  else if (dtype == 1)
+    scan_gate_kernel<bf16_t><<<grid, 256, 0, stream>>>(out, ldo, (const bf16_t*)z, ldz, bias, per_head, head_width, mode,
+                                                       number, first_columns, width);
+  else
+    return fail("scan_gate: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("scan_gate");
+  return 0;
+}
+
+HFEE_API int hfee_linear_scan(float* out, int64_t ldo, float* state, const float* q, int64_t ldq, const float* k,
+                              int64_t ldk, const float* v, int64_t ldv, const float* decay, int64_t ldd,
+                              const float* beta, int64_t ldb, const int* segment_rows, const int* segment_lengths,
+                              const int* segment_slots, int segments, int heads, int qk_heads, int dim, int vdim,
+                              int rule, hipStream_t stream) {
+  HFEE_REQUIRE(segments >= 0 && segments <= 65535, "linear_scan: bad segment count");
+  if (segments == 0) return 0;
+  HFEE_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && heads <= 65535,
+               "linear_scan: %d heads are not a multiple of %d query/key heads", heads, qk_heads);
+  HFEE_REQUIRE(dim >= 1 && dim <= 512 && vdim >= 1, "linear_scan: key sizes of 1 to 512");
+  HFEE_REQUIRE(rule == 0 || (rule == 1 && beta != nullptr), "linear_scan: rule 0, or rule 1 with its writing strengths");
+  HFEE_REQUIRE(ldq >= (int64_t)qk_heads * dim && ldk >= (int64_t)qk_heads * dim && ldv >= (int64_t)heads * vdim &&
+               ldd >= (int64_t)heads * dim && ldo >= (int64_t)heads * vdim, "linear_scan: rows too short");
+  dim3 grid((vdim + 15) / 16, heads, segments);
+  const int per = (dim + 3) / 4;
+#define LAUNCH(DPT, RULE)                                                                                             \
+  linear_scan_kernel<DPT, RULE><<<grid, 64, 0, stream>>>(out, ldo, state, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, \
+      segment_rows, segment_lengths, segment_slots, heads, qk_heads, dim, vdim)
+#define PICK(RULE)                                                                                                    \
+  if (per <= 4) LAUNCH(4, RULE); else if (per <= 8) LAUNCH(8, RULE); else if (per <= 16) LAUNCH(16, RULE);            \
+  else if (per <= 32) LAUNCH(32, RULE); else if (per <= 64) LAUNCH(64, RULE); else LAUNCH(128, RULE)
+  if (rule == 0) { PICK(0); } else { PICK(1); }
+#undef PICK
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("linear_scan");
+  return 0;
+}
+
+HFEE_API int hfee_head_norm_gate(void* out, int64_t ldo, const float* o, int64_t ldi, const void* gate, int64_t ldg,
+                                 int dtype, const float* weight, int heads, int vdim, float eps, int act, int n,
+                                 hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && heads > 0 && vdim > 0 && (act == 0 || act == 1), "head_norm_gate: bad sizes");
+  HFEE_REQUIRE(ldo >= (int64_t)heads * vdim && ldi >= (int64_t)heads * vdim && ldg >= (int64_t)heads * vdim,
+               "head_norm_gate: rows too short");
+  if (n == 0) return 0;
+  const int64_t items = (int64_t)n * heads;
+  const unsigned blocks = (unsigned)((items + 3) / 4);
+  if (dtype == 0)
+    head_norm_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, ldo, o, ldi, (const float*)gate, ldg, weight,
+                                                            heads, vdim, eps, act, n);
+  else if (dtype == 1)
+    head_norm_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, ldo, o, ldi, (const bf16_t*)gate, ldg, weight,
+                                                             heads, vdim, eps, act, n);
+  else
+    return fail("head_norm_gate: unknown dtype %d", dtype);
+  HFEE_CHECK_LAUNCH("head_norm_gate");
+  return 0;
+}

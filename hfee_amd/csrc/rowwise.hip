@@ -6,6 +6,7 @@
 //                  next[r] = x[r] / sqrt(mean(x[r]^2) + eps2) * w2
 //   bias_act:      out = act(in + bias)
 //   rmsnorm_cols:  a norm over a block of columns of rows in the engine's dtype (a latent's norm)
+//   layernorm:     out[r] = (x[r] - mean) / sqrt(mean((x[r] - mean)^2) + eps) * w, no bias
 //
 // All sums in float32, one workgroup a row, a fixed order of additions.
 #include "common.h"
@@ -14,10 +15,12 @@ using namespace hfee;
 
 namespace {
 
-enum { ACT_NONE = 0, ACT_RELU2 = 1, ACT_RELU = 2, ACT_GELU_TANH = 3, ACT_SILU = 4 };
+enum { ACT_NONE = 0, ACT_RELU2 = 1, ACT_RELU = 2, ACT_GELU_TANH = 3, ACT_SILU = 4, ACT_XIELU = 5 };
 
-__device__ __forceinline__ float activate(float z, int act) {
+// ACT_XIELU has two numbers: a z^2 + z / 2 above zero, b (exp(z) - 1 - z) + z / 2 at and below it.
+__device__ __forceinline__ float activate(float z, int act, float a = 0.f, float b = 0.f) {
   switch (act) {
+    case ACT_XIELU: return z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
     case ACT_RELU2: { const float r = fmaxf(z, 0.f); return r * r; }
     case ACT_RELU: return fmaxf(z, 0.f);
     case ACT_GELU_TANH: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
@@ -122,17 +125,17 @@ __global__ __launch_bounds__(1024) void norm_add_rows_kernel(
 
 template <typename T>
 __global__ void bias_act_kernel(T* __restrict__ out, int64_t ldo, const T* __restrict__ in, int64_t ldi,
-                                const T* __restrict__ bias, int width, int act) {
+                                const T* __restrict__ bias, int width, int act, float pa, float pb) {
   const int64_t row = blockIdx.y;
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= width) return;
   const float z = to_float<T>(in[row * ldi + j]) + (bias ? to_float<T>(bias[j]) : 0.f);
-  out[row * ldo + j] = from_float<T>(activate(z, act));
+  out[row * ldo + j] = from_float<T>(activate(z, act, pa, pb));
 }
 
 // eight bfloat16 values a thread (16 bytes), for widths that are multiples of 8 and aligned rows
 __global__ void bias_act_bf16x8_kernel(bf16_t* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ in, int64_t ldi,
-                                       const bf16_t* __restrict__ bias, int width, int act) {
+                                       const bf16_t* __restrict__ bias, int width, int act, float pa, float pb) {
   typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
   const int64_t row = blockIdx.y;
   const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
@@ -143,8 +146,8 @@ __global__ void bias_act_bf16x8_kernel(bf16_t* __restrict__ out, int64_t ldo, co
   u32x4_t o;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const float lo = activate(bf16_to_float((bf16_t)(v[i] & 0xffff)) + bf16_to_float((bf16_t)(b[i] & 0xffff)), act);
-    const float hi = activate(bf16_to_float((bf16_t)(v[i] >> 16)) + bf16_to_float((bf16_t)(b[i] >> 16)), act);
+    const float lo = activate(bf16_to_float((bf16_t)(v[i] & 0xffff)) + bf16_to_float((bf16_t)(b[i] & 0xffff)), act, pa, pb);
+    const float hi = activate(bf16_to_float((bf16_t)(v[i] >> 16)) + bf16_to_float((bf16_t)(b[i] >> 16)), act, pa, pb);
     o[i] = (uint32_t)float_to_bf16(lo) | ((uint32_t)float_to_bf16(hi) << 16);
   }
   *reinterpret_cast<u32x4_t*>(out + row * ldo + j) = o;
@@ -169,7 +172,45 @@ __global__ __launch_bounds__(256) void rmsnorm_cols_kernel(T* __restrict__ out, 
     orow[j] = from_float<T>(to_float<T>(xr[j]) * inv * weight_at<TW>(w, j, offset));
 }
 
+// x float32 [rows, d]; row r of out is made from row rows[r] (or r) of x.  The mean first, then the
+// mean of the squared deviations from it, both as sums over the workgroup in a fixed order.
+template <typename TO, typename TW>
+__global__ __launch_bounds__(256) void layernorm_kernel(TO* __restrict__ out, const float* __restrict__ x,
+                                                        const TW* __restrict__ w, const int* __restrict__ rows,
+                                                        float eps, int d) {
+  __shared__ float scratch[16];
+  const int64_t r = blockIdx.x;
+  const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
+  float sum = 0.f;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) sum += xr[j];
+  const float mean = block_sum(sum, scratch) / (float)d;
+  float ss = 0.f;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) {
+    const float v = xr[j] - mean;
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)d + eps);
+  TO* o = out + r * d;
+  for (int j = threadIdx.x; j < d; j += blockDim.x) o[j] = from_float<TO>((xr[j] - mean) * inv * to_float<TW>(w[j]));
+}
+
 }  // namespace
+
+HFEE_API int hfee_layernorm(void* out, int out_dtype, const float* x, const void* w, int w_dtype, const int* rows,
+                            float eps, int n, int d, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && d > 0, "layernorm: bad sizes n=%d d=%d", n, d);
+  HFEE_REQUIRE(eps >= 0.f, "layernorm: eps must not be negative");
+  if (n == 0) return 0;
+#define LAUNCH(TO, TW) layernorm_kernel<TO, TW><<<n, 256, 0, stream>>>((TO*)out, x, (const TW*)w, rows, eps, d)
+  if (out_dtype == 0 && w_dtype == 0) LAUNCH(float, float);
+  else if (out_dtype == 0 && w_dtype == 1) LAUNCH(float, bf16_t);
+  else if (out_dtype == 1 && w_dtype == 0) LAUNCH(bf16_t, float);
+  else if (out_dtype == 1 && w_dtype == 1) LAUNCH(bf16_t, bf16_t);
+  else return fail("layernorm: unknown dtypes");
+#undef LAUNCH
+  HFEE_CHECK_LAUNCH("layernorm");
+  return 0;
+}
 
 // y_dtype / bias_dtype / w_dtype / next_dtype: 0 float32, 1 bfloat16.
 HFEE_API int hfee_norm_add(float* x, const void* y, int y_dtype, const void* bias, int bias_dtype, const void* w,
@@ -229,9 +270,9 @@ HFEE_API int hfee_norm_add(float* x, const void* y, int y_dtype, const void* bia
 }
 
 HFEE_API int hfee_bias_act(void* out, int64_t ldo, const void* in, int64_t ldi, const void* bias, int dtype, int n,
-                           int width, int act, hipStream_t stream) {
+                           int width, int act, float pa, float pb, hipStream_t stream) {
   HFEE_REQUIRE(n >= 0 && width > 0, "bias_act: bad sizes");
-  HFEE_REQUIRE(act >= ACT_NONE && act <= ACT_SILU, "bias_act: unknown activation %d", act);
+  HFEE_REQUIRE(act >= ACT_NONE && act <= ACT_XIELU, "bias_act: unknown activation %d", act);
   HFEE_REQUIRE(n <= 65535 * 32, "bias_act: too many rows");
   if (n == 0) return 0;
   const bool wide = dtype == 1 && width % 8 == 0 && ldo % 8 == 0 && ldi % 8 == 0 &&
@@ -241,13 +282,13 @@ HFEE_API int hfee_bias_act(void* out, int64_t ldo, const void* in, int64_t ldi, 
     dim3 grid((width + 255) / 256, rows);
     if (wide)
       bias_act_bf16x8_kernel<<<dim3((width / 8 + 255) / 256, rows), 256, 0, stream>>>(
-          (bf16_t*)out + (int64_t)r0 * ldo, ldo, (const bf16_t*)in + (int64_t)r0 * ldi, ldi, (const bf16_t*)bias, width, act);
+          (bf16_t*)out + (int64_t)r0 * ldo, ldo, (const bf16_t*)in + (int64_t)r0 * ldi, ldi, (const bf16_t*)bias, width, act, pa, pb);
     else if (dtype == 0)
       bias_act_kernel<float><<<grid, 256, 0, stream>>>((float*)out + (int64_t)r0 * ldo, ldo, (const float*)in + (int64_t)r0 * ldi,
-                                                        ldi, (const float*)bias, width, act);
+                                                        ldi, (const float*)bias, width, act, pa, pb);
     else if (dtype == 1)
       bias_act_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out + (int64_t)r0 * ldo, ldo, (const bf16_t*)in + (int64_t)r0 * ldi,
-                                                         ldi, (const bf16_t*)bias, width, act);
+                                                         ldi, (const bf16_t*)bias, width, act, pa, pb);
     else
       return fail("bias_act: unknown dtype %d", dtype);
   }

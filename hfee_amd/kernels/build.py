@@ -33,7 +33,8 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-fvisibility=h
          "-Wno-unused-command-line-argument"]
 
 CORE_SOURCES = ["elementwise.hip", "gemm_f32.hip", "attention_ref.hip", "gemm_bf16.hip", "gemm_skinny.hip",
-                "sampling.hip", "random_fill.hip", "yardstick.hip", "attention_kv.hip", "rowwise.hip"]
+                "sampling.hip", "random_fill.hip", "yardstick.hip", "attention_kv.hip", "rowwise.hip", "attention_mix.hip",
+                "recurrent.hip", "moe.hip"]
 ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
 ATTENTION_KV_SOURCE = "attention_kv_bf16.hip"      # compiled per (key size, value size)

@@ -23,7 +23,7 @@ class KernelError(RuntimeError):
 P, I, L, F, D, U64 = c_void_p, c_int, c_int64, c_float, c_double, c_uint64
 
 _CORE_SIGNATURES = {
-    "hfee_embed": [P, P, I, P, I, I, P],
+    "hfee_embed": [P, P, I, P, I, I, F, P],
     "hfee_embed_emit": [P, P, P, I, I, P, I, P, L, P, L, P],
     "hfee_rmsnorm": [P, I, P, P, I, P, F, I, I, P],
     "hfee_cast_rows": [P, I, P, P, I, I, P],
@@ -51,7 +51,18 @@ _CORE_SIGNATURES = {
     "hfee_attention_kv_plain": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, I, F, P, I, P],
     "hfee_head_linear": [P, L, L, P, L, L, P, I, I, I, I, I, I, P],
     "hfee_norm_add": [P, P, I, P, I, P, I, F, F, P, I, P, F, I, I, P],
-    "hfee_bias_act": [P, L, P, L, P, I, I, I, I, P],
+    "hfee_bias_act": [P, L, P, L, P, I, I, I, I, F, F, P],
+    "hfee_layernorm": [P, I, P, P, I, P, F, I, I, P],
+    "hfee_attention_mix_prepare": [P, L, P, L, I, I, I, I, P, P, P, I, P, P, I, I, I, I, F, P, I, I, P],
+    "hfee_attention_mix": [P, L, P, L, P, I, P, P, P, I, I, I, I, I, F, P, I, I, P, I, P],
+    "hfee_short_conv_silu": [P, L, P, L, P, I, P, P, P, P, I, I, I, P],
+    "hfee_short_conv_keep": [P, P, L, I, P, P, P, I, I, I, P],
+    "hfee_unit_heads": [P, L, I, I, F, F, I, P],
+    "hfee_scan_gate": [P, L, P, L, I, P, P, I, I, F, I, I, I, P],
+    "hfee_linear_scan": [P, L, P, P, L, P, L, P, L, P, L, P, L, P, P, P, I, I, I, I, I, I, P],
+    "hfee_head_norm_gate": [P, L, P, L, P, L, I, P, I, I, F, I, I, P],
+    "hfee_moe_up": [P, P, L, P, P, I, P, P, P, I, I, I, I, I, P],
+    "hfee_moe_down": [P, L, P, P, I, P, P, P, P, F, I, I, I, I, I, I, P],
     "hfee_rmsnorm_cols": [P, L, P, L, I, P, I, F, F, I, I, P],
 }
 

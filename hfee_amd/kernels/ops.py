@@ -67,8 +67,8 @@ def _i32(t, what, n=None):
 
 # ------------------------------------------------------------------ simple ops
 
-def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, emit: dict | None = None):
-    """out[i, :] = table[ids[i], :] as float32.
+def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, emit: dict | None = None, scale: float = 1.0):
+    """out[i, :] = table[ids[i], :] * scale as float32.
 
     emit: dict(weight, out, shares) as for `linear_fused`: the first half of the norm that
     follows, bfloat16(out * weight) into emit["out"] and the rows' sums of squares in
@@ -80,8 +80,9 @@ def embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, emit: dict 
     _check(table.dim() == 2 and table.is_contiguous() and table.shape[1] == d, "embed: table shape")
     _i32(ids, "embed ids", n)
     if emit is None:
-        lib.core().call("hfee_embed", _ptr(out), _ptr(table), _dt(table), _ptr(ids), n, d, _stream())
+        lib.core().call("hfee_embed", _ptr(out), _ptr(table), _dt(table), _ptr(ids), n, d, float(scale), _stream())
         return
+    _check(scale == 1.0, "embed: a scaled lookup does not begin the norm that follows")
     eo, es, ew = emit["out"], emit["shares"], emit["weight"]
     _gpu(eo, es, ew)
     _check(can_embed_emit(table, n), "embed: the norm's first half only with a bfloat16 table of a width that is a "
@@ -930,7 +931,7 @@ def head_linear(out, x, weight, heads: int, n_in: int, n_out: int, tail: int = 0
 
 # ----------------------------------------------- blocks that norm a sub-layer's output; biases
 
-ROW_ACTIVATIONS = {"none": 0, "relu2": 1, "relu": 2, "gelu_tanh": 3, "silu": 4}
+ROW_ACTIVATIONS = {"none": 0, "relu2": 1, "relu": 2, "gelu_tanh": 3, "silu": 4, "xielu": 5}
 
 
 def norm_add(x, y, weight, eps: float, bias=None, next_out=None, next_weight=None, next_eps: float = 0.0):
@@ -953,8 +954,9 @@ def norm_add(x, y, weight, eps: float, bias=None, next_out=None, next_weight=Non
                     _ptr(next_weight), float(next_eps), n, d, _stream())
 
 
-def bias_act(out, x, bias, activation: str = "none"):
-    """out = activation(x + bias), row by row; "relu2" is the square of relu."""
+def bias_act(out, x, bias, activation: str = "none", numbers=(0.0, 0.0)):
+    """out = activation(x + bias), row by row; "relu2" is the square of relu; "xielu" with its two
+    `numbers` (a, b) is a z^2 + z / 2 above zero and b (exp(z) - 1 - z) + z / 2 at and below it."""
     _gpu(out, x, bias)
     _check(activation in ROW_ACTIVATIONS, f"bias_act: the activations are {sorted(ROW_ACTIVATIONS)}, not {activation!r}")
     n, w, ldi = _rows2d(x, "bias_act x")
@@ -963,7 +965,7 @@ def bias_act(out, x, bias, activation: str = "none"):
     if bias is not None:
         _check(bias.numel() == w and bias.is_contiguous() and bias.dtype == x.dtype, "bias_act: bias")
     lib.core().call("hfee_bias_act", _ptr(out), ldo, _ptr(x), ldi, _ptr(bias), _dt(x), n, w, ROW_ACTIVATIONS[activation],
-                    _stream())
+                    float(numbers[0]), float(numbers[1]), _stream())
 
 
 def rmsnorm_cols(out, x, weight, eps: float):
@@ -976,3 +978,260 @@ def rmsnorm_cols(out, x, weight, eps: float):
     _check(weight.numel() == w and weight.is_contiguous(), "rmsnorm_cols: weight width")
     lib.core().call("hfee_rmsnorm_cols", _ptr(out), ldo, _ptr(x), ldx, _dt(x), _ptr(weight), _dt(weight), 0.0, float(eps),
                     n, w, _stream())
+
+
+def layernorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None):
+    """out[r] = (x[rows[r] or r] - mean) / sqrt(variance + eps) * weight, the variance the mean of the
+    squared deviations; x float32, no bias."""
+    _gpu(out, x, weight, rows)
+    n, d, _ = _rows2d(out, "layernorm out")
+    _check(out.is_contiguous() and x.is_contiguous() and x.dtype == torch.float32, "layernorm: contiguous float32 x")
+    _check(x.dim() == 2 and x.shape[1] == d, "layernorm: width mismatch")
+    _check(weight.numel() == d and weight.is_contiguous(), "layernorm: weight width mismatch")
+    if rows is None:
+        _check(x.shape[0] >= n, "layernorm: fewer input rows than output rows")
+    else:
+        _i32(rows, "layernorm rows", n)
+    lib.core().call("hfee_layernorm", _ptr(out), _dt(out), _ptr(x), _ptr(weight), _dt(weight), _ptr(rows), float(eps),
+                    n, d, _stream())
+
+
+# --------------------------------- attention whose heads' scores are mixed, over keys that are the values
+
+def _mix_cache(cache_layer, kv_heads, dim, page_size, what):
+    _check(cache_layer.is_contiguous() and cache_layer.dim() == 4 and
+           tuple(cache_layer.shape[1:]) == (kv_heads, page_size, 2 * dim),
+           f"{what}: the cache layer must be [pages, kv_heads, page_size, 2 * dim]")
+
+
+def _tables(block_tables, what):
+    _check(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1, f"{what}: block tables")
+
+
+def attention_mix_prepare(q, k, positions, token_segment, block_tables, cos, sin, cache_layer, num_heads: int,
+                          kv_heads: int, dim: int, page_size: int, max_position: int, norm: bool = True,
+                          eps: float = 0.0):
+    """q ([n, num_heads * dim], in place) and k ([n, kv_heads * dim]) rotated in their first 2 * half
+    dims (cos/sin float32 [positions, half], pairs (i, i + half)) and then, with `norm`, divided by
+    their root mean square over each head; the key as it is scored and the key as it was projected
+    go into the token's slot of `cache_layer` ([pages, kv_heads, page_size, 2 * dim]).  k None: only
+    q is made ready."""
+    _gpu(q, k, positions, cos, sin, cache_layer)
+    some = q if q is not None else k
+    _check(some is not None, "attention_mix_prepare: nothing to do")
+    n = some.shape[0]
+    ldq = ldk = 0
+    if q is not None:
+        nq, wq, ldq = _rows2d(q, "attention_mix_prepare q")
+        _check(wq == num_heads * dim, "attention_mix_prepare: q shape")
+    if k is not None:
+        nk, wk, ldk = _rows2d(k, "attention_mix_prepare k")
+        _check(nk == n and wk == kv_heads * dim and k.dtype == cache_layer.dtype and (q is None or q.dtype == k.dtype),
+               "attention_mix_prepare: k shape or dtype")
+        _mix_cache(cache_layer, kv_heads, dim, page_size, "attention_mix_prepare")
+        _i32(token_segment, "attention_mix_prepare token_segment", n)
+        _tables(block_tables, "attention_mix_prepare")
+    _i32(positions, "attention_mix_prepare positions", n)
+    half = table_positions = 0
+    if cos is not None:
+        _check(cos.shape == sin.shape and cos.dim() == 2 and cos.is_contiguous() and sin.is_contiguous()
+               and cos.dtype == sin.dtype == torch.float32, "attention_mix_prepare: cos/sin tables")
+        table_positions, half = cos.shape
+    has_k = k is not None
+    lib.core().call("hfee_attention_mix_prepare", _ptr(q), ldq, _ptr(k), ldk, _dt(some), num_heads, kv_heads, dim,
+                    _ptr(positions), _ptr(token_segment if has_k else None), _ptr(block_tables if has_k else None),
+                    block_tables.stride(0) if has_k else 0, _ptr(cos), _ptr(sin), half, table_positions,
+                    int(max_position), 1 if norm else 0, float(eps), _ptr(cache_layer if has_k else None), page_size, n,
+                    _stream())
+
+
+def attention_mix(out, q, cache_layer, positions, token_segment, block_tables, num_heads: int, kv_heads: int, dim: int,
+                  page_size: int, scale: float, mix=None, chunk: int = 0, sink=None):
+    """Token t at position p reads the keys of its sequence from the start of p's chunk (chunk 0: from
+    position 0) up to p; the heads' scores q . k * scale are mixed by `mix` (float32 [heads, heads],
+    score_h = sum_g mix[h, g] score_g; None: not mixed); sink: None, "zero" (one more term exp(0) in
+    the softmax's denominator) or a float32 tensor [heads] of learned scores; the values are the
+    second half of each cache slot."""
+    _gpu(out, q, cache_layer, positions, token_segment, block_tables, mix)
+    n, w, ldq = _rows2d(q, "attention_mix q")
+    no, wo, ldo = _rows2d(out, "attention_mix out")
+    _check(no == n and w == num_heads * dim and wo == num_heads * dim, "attention_mix: q/out shape")
+    _check(q.dtype == out.dtype == cache_layer.dtype, "attention_mix: dtype mismatch")
+    _mix_cache(cache_layer, kv_heads, dim, page_size, "attention_mix")
+    _i32(positions, "attention_mix positions", n)
+    _i32(token_segment, "attention_mix token_segment", n)
+    _tables(block_tables, "attention_mix")
+    if mix is not None:
+        _check(mix.dtype == torch.float32 and mix.is_contiguous() and tuple(mix.shape) == (num_heads, num_heads),
+               "attention_mix: mix must be float32 [heads, heads]")
+    sinks, mode = None, 0
+    if isinstance(sink, str):
+        _check(sink == "zero", "attention_mix: sink is None, 'zero' or a tensor")
+        mode = 1
+    elif sink is not None:
+        _gpu(sink)
+        _check(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == num_heads,
+               "attention_mix: sinks must be float32 [heads]")
+        sinks, mode = sink, 2
+    lib.core().call("hfee_attention_mix", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _dt(q), _ptr(positions),
+                    _ptr(token_segment), _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, dim, page_size,
+                    float(scale), _ptr(mix), int(chunk), mode, _ptr(sinks), n, _stream())
+
+
+# ------------------------------------------------ mixers with a state of fixed size a request
+
+def _f32rows(t, what):
+    n, w, ld = _rows2d(t, what)
+    _check(t.dtype == torch.float32, f"{what}: float32 expected")
+    return n, w, ld
+
+
+def short_conv_silu(y, x, state, taps, token_segment, segment_rows, segment_slots):
+    """y (float32 [n, C]) = silu of the causal convolution of x ([n, C], the step's rows) with taps
+    (float32 [C, K], the last column the current token's) per channel; the K - 1 inputs before a
+    portion's first token come from state[slot] ([slots, K - 1, C] in x's dtype, the newest last)."""
+    _gpu(y, x, state, taps, token_segment, segment_rows, segment_slots)
+    n, C, ldx = _rows2d(x, "short_conv_silu x")
+    ny, wy, ldy = _f32rows(y, "short_conv_silu y")
+    K = taps.shape[1]
+    _check(ny == n and wy == C and tuple(taps.shape) == (C, K) and taps.dtype == torch.float32 and taps.is_contiguous(),
+           "short_conv_silu: shapes of y and taps")
+    _check(state.dtype == x.dtype and state.is_contiguous() and tuple(state.shape[1:]) == (K - 1, C),
+           "short_conv_silu: the state must be [slots, K - 1, C] in x's dtype")
+    _i32(token_segment, "short_conv_silu token_segment", n)
+    _i32(segment_rows, "short_conv_silu segment_rows")
+    _i32(segment_slots, "short_conv_silu segment_slots")
+    lib.core().call("hfee_short_conv_silu", _ptr(y), ldy, _ptr(x), ldx, _ptr(state), _dt(x), _ptr(taps),
+                    _ptr(token_segment), _ptr(segment_rows), _ptr(segment_slots), C, K, n, _stream())
+
+
+def short_conv_keep(state, x, segment_rows, segment_lengths, segment_slots):
+    """state[slot] <- the last K - 1 inputs of each segment's sequence (the step's rows x, and what the
+    state held before where a portion is shorter than K - 1)."""
+    _gpu(state, x, segment_rows, segment_lengths, segment_slots)
+    n, C, ldx = _rows2d(x, "short_conv_keep x")
+    _check(state.dtype == x.dtype and state.is_contiguous() and state.dim() == 3 and state.shape[2] == C,
+           "short_conv_keep: the state must be [slots, K - 1, C] in x's dtype")
+    segments = segment_rows.numel()
+    _i32(segment_rows, "short_conv_keep segment_rows")
+    _i32(segment_lengths, "short_conv_keep segment_lengths", segments)
+    _i32(segment_slots, "short_conv_keep segment_slots", segments)
+    lib.core().call("hfee_short_conv_keep", _ptr(state), _ptr(x), ldx, _dt(x), _ptr(segment_rows), _ptr(segment_lengths),
+                    _ptr(segment_slots), C, state.shape[1] + 1, segments, _stream())
+
+
+def unit_heads(x, heads: int, dim: int, eps: float, factor: float = 1.0):
+    """x (float32 [n, heads * dim], in place) <- x / sqrt(sum(x^2) + eps) * factor over each head."""
+    _gpu(x)
+    n, w, ldx = _f32rows(x, "unit_heads x")
+    _check(w == heads * dim, "unit_heads: width")
+    lib.core().call("hfee_unit_heads", _ptr(x), ldx, heads, dim, float(eps), float(factor), n, _stream())
+
+
+SCAN_GATES = {"step_decay": 0, "root_sigmoid": 1, "sigmoid": 2, "cast": 3}
+
+
+def scan_gate(out, z, kind: str, bias=None, per_head=None, head_width: int = 0, number: float = 1.0, first_columns: int = 0):
+    """out (float32) from a projection z (engine dtype), column by column:
+    "step_decay": exp(-exp(per_head[column // head_width]) * softplus(z + bias));
+    "root_sigmoid": sigmoid(z + bias) ** (1 / number);  "sigmoid": sigmoid(z + bias);
+    "cast": z * number in the first `first_columns` columns, z in the others."""
+    _gpu(out, z, bias, per_head)
+    n, w, ldz = _rows2d(z, "scan_gate z")
+    no, wo, ldo = _f32rows(out, "scan_gate out")
+    _check(kind in SCAN_GATES and no == n and wo == w, "scan_gate: kind or shapes")
+    for t, what in ((bias, "bias"), (per_head, "per_head")):
+        if t is not None:
+            _check(t.dtype == torch.float32 and t.is_contiguous(), f"scan_gate: {what} must be contiguous float32")
+    if bias is not None:
+        _check(bias.numel() == w, "scan_gate: bias width")
+    if kind == "step_decay":
+        _check(per_head is not None and head_width > 0 and per_head.numel() * head_width == w, "scan_gate: one number a head")
+    lib.core().call("hfee_scan_gate", _ptr(out), ldo, _ptr(z), ldz, _dt(z), _ptr(bias), _ptr(per_head), int(head_width),
+                    SCAN_GATES[kind], float(number), int(first_columns), n, w, _stream())
+
+
+def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots, heads: int,
+                qk_heads: int, dim: int, vdim: int, rule: str):
+    """Walks each segment's rows in order from state[slot] ([slots, heads, dim, vdim] float32, updated in
+    place).  rule "decay_add": S <- diag(decay) S + k v^T; "delta": S <- diag(decay) S,
+    S <- S + k (beta (v - S^T k))^T; out = S^T q.  q, k: float32 [n, qk_heads * dim] (head h reads
+    q/k head h // (heads / qk_heads)); v, out: [n, heads * vdim]; decay: [n, heads * dim]; beta [n, heads]."""
+    _gpu(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots)
+    n, wq, ldq = _f32rows(q, "linear_scan q")
+    nk, wk, ldk = _f32rows(k, "linear_scan k")
+    nv, wv, ldv = _f32rows(v, "linear_scan v")
+    nd, wd, ldd = _f32rows(decay, "linear_scan decay")
+    no, wo, ldo = _f32rows(out, "linear_scan out")
+    _check(rule in ("decay_add", "delta"), "linear_scan: rule is 'decay_add' or 'delta'")
+    _check(nk == nv == nd == no == n and wq == wk == qk_heads * dim and wv == wo == heads * vdim and wd == heads * dim,
+           "linear_scan: shapes")
+    _check(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dim, vdim),
+           "linear_scan: the state must be float32 [slots, heads, dim, vdim]")
+    ldb = 0
+    if rule == "delta":
+        nb, wb, ldb = _f32rows(beta, "linear_scan beta")
+        _check(nb == n and wb == heads, "linear_scan: beta [n, heads]")
+    segments = segment_rows.numel()
+    _i32(segment_rows, "linear_scan segment_rows")
+    _i32(segment_lengths, "linear_scan segment_lengths", segments)
+    _i32(segment_slots, "linear_scan segment_slots", segments)
+    lib.core().call("hfee_linear_scan", _ptr(out), ldo, _ptr(state), _ptr(q), ldq, _ptr(k), ldk, _ptr(v), ldv, _ptr(decay),
+                    ldd, _ptr(beta if rule == "delta" else None), ldb, _ptr(segment_rows), _ptr(segment_lengths),
+                    _ptr(segment_slots), segments, heads, qk_heads, dim, vdim, 1 if rule == "delta" else 0, _stream())
+
+
+def head_norm_gate(out, o, gate, weight, heads: int, vdim: int, eps: float, activation: str):
+    """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight * act(gate[t, h]) over each head's vdim
+    values; o float32, gate and out in the engine's dtype, weight float32 [vdim]; act "sigmoid" or "silu"."""
+    _gpu(out, o, gate, weight)
+    n, w, ldi = _f32rows(o, "head_norm_gate o")
+    ng, wg, ldg = _rows2d(gate, "head_norm_gate gate")
+    no, wo, ldo = _rows2d(out, "head_norm_gate out")
+    _check(ng == no == n and wg == wo == w == heads * vdim and gate.dtype == out.dtype, "head_norm_gate: shapes and dtypes")
+    _check(weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() == vdim, "head_norm_gate: weight float32 [vdim]")
+    _check(activation in ("sigmoid", "silu"), "head_norm_gate: the gate's activation is 'sigmoid' or 'silu'")
+    lib.core().call("hfee_head_norm_gate", _ptr(out), ldo, _ptr(o), ldi, _ptr(gate), ldg, _dt(out), _ptr(weight), heads, vdim,
+                    float(eps), 0 if activation == "sigmoid" else 1, n, _stream())
+
+
+# ------------------------------------------------------------------ experts
+
+def _experts_of(chosen, table, token_ids, n, top, what):
+    if chosen is not None:
+        _check(chosen.dtype == torch.int32 and chosen.is_contiguous() and tuple(chosen.shape) == (n, top), f"{what}: chosen int32 [n, top]")
+        return
+    _check(table is not None and token_ids is not None and table.dtype == torch.int32 and table.is_contiguous()
+           and table.dim() == 2 and table.shape[1] == top, f"{what}: a table int32 [vocabulary, top] and the token ids")
+    _i32(token_ids, f"{what} token_ids", n)
+
+
+def moe_up(act, h, w_gate, w_up, top: int, chosen=None, table=None, token_ids=None):
+    """act[t * top + j] = silu(w_gate[e] @ h[t]) * (w_up[e] @ h[t]), e the j-th expert of token t
+    (chosen[t, j], or table[token_ids[t], j]); w_gate, w_up: [experts, ff, width]."""
+    _gpu(act, h, w_gate, w_up, chosen, table, token_ids)
+    n, width, ldh = _rows2d(h, "moe_up h")
+    E, F, W = w_gate.shape
+    _check(W == width and w_up.shape == w_gate.shape and w_gate.is_contiguous() and w_up.is_contiguous(), "moe_up: weights [experts, ff, width]")
+    _check(act.is_contiguous() and tuple(act.shape) == (n * top, F) and act.dtype == h.dtype == w_gate.dtype == w_up.dtype,
+           "moe_up: act [n * top, ff], one dtype")
+    _experts_of(chosen, table, token_ids, n, top, "moe_up")
+    lib.core().call("hfee_moe_up", _ptr(act), _ptr(h), ldh, _ptr(w_gate), _ptr(w_up), _dt(h), _ptr(chosen), _ptr(table),
+                    _ptr(token_ids), top, E, F, width, n, _stream())
+
+
+def moe_down(x, act, w_down, top: int, weight: float = 1.0, pair_weights=None, chosen=None, table=None, token_ids=None,
+             accumulate: bool = True):
+    """x[t] (+)= sum_j weight_tj * (w_down[e_j] @ act[t * top + j]); x float32 [n, width], w_down
+    [experts, width, ff]; weight_tj = pair_weights[t, j] (float32) or the one number `weight`."""
+    _gpu(x, act, w_down, pair_weights, chosen, table, token_ids)
+    n, width, ldx = _f32rows(x, "moe_down x")
+    E, W, F = w_down.shape
+    _check(W == width and w_down.is_contiguous() and act.is_contiguous() and tuple(act.shape) == (n * top, F)
+           and act.dtype == w_down.dtype, "moe_down: w_down [experts, width, ff], act [n * top, ff]")
+    if pair_weights is not None:
+        _check(pair_weights.dtype == torch.float32 and pair_weights.is_contiguous() and tuple(pair_weights.shape) == (n, top),
+               "moe_down: pair_weights float32 [n, top]")
+    _experts_of(chosen, table, token_ids, n, top, "moe_down")
+    lib.core().call("hfee_moe_down", _ptr(x), ldx, _ptr(act), _ptr(w_down), _dt(act), _ptr(chosen), _ptr(table),
+                    _ptr(token_ids), _ptr(pair_weights), float(weight), top, E, F, width, 1 if accumulate else 0, n, _stream())

@@ -8,6 +8,10 @@ x += norm_b(mixer(norm_a(x))); x += norm_d(feed_forward(norm_c(x))), with four n
 weights, and a layer may have no feed-forward.  The sub-layers write float32 rows
 (`forward_into`); one launch norms them, adds them to the stream and makes the norm of the new
 stream for whatever follows (`ops.norm_add`), across layers too.
+
+"parallel" has one norm whose output both sub-layers read: with h = norm(x),
+x += mixer(h) + feed_forward(h).  Both add their last product straight into the float32 stream, the
+mixer first; a layer may have no feed-forward.
 """
 from __future__ import annotations
 
@@ -158,3 +162,44 @@ class SandwichBlock(Part):
         self._add_normed(ctx, x, y, self.mixer_post_norm, getattr(self.mixer, "output_bias", None), h2)
         y = self._rows_of(self.feed_forward, ctx, h2, self.hidden)
         self._add_normed(ctx, x, y, self.feed_forward_post_norm, getattr(self.feed_forward, "output_bias", None), h_next)
+
+
+@register_block("parallel")
+class ParallelBlock(Part):
+    """Tensor names by role: mixer_norm (the whole name behind the layer's prefix), mixer and
+    feed_forward (prefixes)."""
+
+    def __init__(self, spec: LayerSpec, dtype: torch.dtype):
+        self.spec, self.dtype, self.hidden = spec, dtype, spec.hidden
+        self.norm = lookup("norm", spec.mixer_norm.kind)(spec.mixer_norm, spec.name_of("mixer_norm", "norm.weight"))
+        self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, spec.name_of("mixer", "mixer."), dtype)
+        self.feed_forward = None
+        if spec.feed_forward is not None:
+            self.feed_forward = lookup("feed_forward", spec.feed_forward.kind)(
+                spec.feed_forward, spec.name_of("feed_forward", "feed_forward."), dtype)
+
+    def _own(self):
+        return [p for p in (self.norm, self.mixer, self.feed_forward) if p is not None]
+
+    def parts(self):
+        return [q for p in self._own() for q in p.parts()]
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def key_layout(self):
+        return getattr(self.mixer, "key_layout", lambda: None)()
+
+    def tensor_specs(self):
+        return [s for p in self._own() for s in p.tensor_specs()]
+
+    def bind(self, tensors):
+        for p in self._own():
+            p.bind(tensors)
+
+    def forward(self, ctx, x, entry):
+        h = ctx.rows("block.normed", self.hidden)
+        self.norm.forward(ctx, h, x)
+        self.mixer.forward_add(ctx, x, h, entry.cache, entry.writes_cache)
+        if self.feed_forward is not None:
+            self.feed_forward.forward_add(ctx, x, h)

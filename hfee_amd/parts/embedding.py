@@ -1,7 +1,8 @@
 """Token embedding and the output head.
 
 Embedding: a row gather into the float32 residual stream, no scaling
-(/root/reference/internal/llm/forward.go:75-77).  Head: final norm and the
+(/root/reference/internal/llm/forward.go:75-77) unless the spec gives a `scale`, by which every
+element is multiplied in float32 on its way.  Head: final norm and the
 vocabulary product only for the rows whose logits are wanted
 (/root/reference/internal/llm/forward.go:117-141); it shares the embedding table
 when the model has no separate head (/root/reference/internal/llm/model.go:118-121).
@@ -24,6 +25,7 @@ class Embedding(Part):
 
     def __init__(self, spec: EmbeddingSpec, name: str, vocab: int, hidden: int, dtype: torch.dtype = None):
         self.name, self.vocab, self.hidden = name, vocab, hidden
+        self.scale = float(spec.get("scale", 1.0))
         self.table = None
 
     def tensor_specs(self):
@@ -38,9 +40,9 @@ class Embedding(Part):
 
     def forward(self, ctx, x, then=None):
         emit = None
-        if then is not None and ops.can_embed_emit(self.table, ctx.n):
+        if then is not None and self.scale == 1.0 and ops.can_embed_emit(self.table, ctx.n):
             emit = then.offer(blocks=ops.embed_emit_blocks(self.hidden))
-        ops.embed(x, self.table, ctx.token_ids, emit=emit)
+        ops.embed(x, self.table, ctx.token_ids, emit=emit, scale=self.scale)
 
 
 @register_head("norm_linear")

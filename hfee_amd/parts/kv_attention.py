@@ -89,14 +89,17 @@ def tiles_of(dtype, *weights):
     return ops.tile_weights_if_room(*weights) or (None,) * len(weights)
 
 
-def product(ctx, out, x, weight, tiles=None) -> None:
-    """out = x @ weight.T: up to 64 rows stream the weight's tiles, more go through the tiled kernels."""
+def product(ctx, out, x, weight, tiles=None, add: bool = False) -> None:
+    """out = x @ weight.T: up to 64 rows stream the weight's tiles, more go through the tiled kernels.
+    add: out (float32, the residual stream) += the product."""
     n = x.shape[0]
-    if tiles is not None and n <= ops.SKINNY_MAX_ROWS:
-        ops.linear_fused(out, x, tiles, "f32" if out.dtype == torch.float32 else "bf16",
+    # (the kernels that stream tiles load 16 bytes a lane: a block of columns of a wider buffer must start and
+    # repeat at such a place)
+    if tiles is not None and n <= ops.SKINNY_MAX_ROWS and x.data_ptr() % 16 == 0 and (n == 1 or x.stride(0) % 8 == 0):
+        ops.linear_fused(out, x, tiles, "add" if add else "f32" if out.dtype == torch.float32 else "bf16",
                          **ctx.workspace.product_scratch(n, tiles))
     else:
-        ops.linear(out, x, weight, **ctx.workspace.split_scratch(n, weight))
+        ops.linear(out, x, weight, accumulate=add, **ctx.workspace.split_scratch(n, weight))
 
 
 class _KvMixer(Mixer):

@@ -7,7 +7,9 @@ product's epilogue (and a step of at most 64 tokens folds the norm in front of i
 the same launch).
 
 "dense_mlp" is the feed-forward without a gate: down(activation(up(h) + b_up)) + b_down, the
-activation one of `ops.ROW_ACTIVATIONS` ("relu2": the square of relu), the biases optional.  It
+activation one of `ops.ROW_ACTIVATIONS` ("relu2": the square of relu; "xielu": with two learned numbers
+p, q of a tensor, softplus(p) z^2 + z / 2 above zero and (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2 at
+and below it), the biases optional.  It
 writes float32 rows (`forward_into`) and leaves the last bias to whoever adds the rows to the
 residual stream (`output_bias`): a block that norms them first folds it into that launch."""
 from __future__ import annotations
@@ -116,7 +118,8 @@ class DenseMLP(FeedForward):
                              f"not {self.activation!r}")
         self.prefix, self.dtype = prefix, dtype
         given = dict(spec.get("names") or ())
-        defaults = dict(up="up_proj.weight", up_bias="up_proj.bias", down="down_proj.weight", down_bias="down_proj.bias")
+        defaults = dict(up="up_proj.weight", up_bias="up_proj.bias", down="down_proj.weight", down_bias="down_proj.bias",
+                        activation="act_fn")
         self.names = {role: prefix + given.get(role, default) for role, default in defaults.items()}
         self.output_bias = None          # float32; added by whoever takes the rows of forward_into
 
@@ -126,6 +129,8 @@ class DenseMLP(FeedForward):
         if self.has_bias:
             specs += [TensorSpec(n["up_bias"], (self.intermediate,), role="vector"),
                       TensorSpec(n["down_bias"], (self.hidden,), role="vector")]
+        if self.activation == "xielu":
+            specs.append(TensorSpec(n["activation"], (2,), role="vector"))
         return specs
 
     def bind(self, tensors):
@@ -133,6 +138,10 @@ class DenseMLP(FeedForward):
         self.w_up, self.w_down = tensors.pop(n["up"]).contiguous(), tensors.pop(n["down"]).contiguous()
         self.up_bias = tensors.pop(n["up_bias"]).to(self.dtype).contiguous() if self.has_bias else None
         self.output_bias = tensors.pop(n["down_bias"]).to(torch.float32).contiguous() if self.has_bias else None
+        self.numbers = (0.0, 0.0)
+        if self.activation == "xielu":      # (two numbers, read once: the kernels take them as arguments)
+            p, q = torch.nn.functional.softplus(tensors.pop(n["activation"]).to(torch.float64).cpu()).tolist()
+            self.numbers = (p, 0.5 + q)
         # a second copy in tiles for steps of up to 64 rows, whose products stream the weights
         self.w_up_tiles = self.w_down_tiles = None
         if self.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.intermediate % 8 == 0:
@@ -151,10 +160,21 @@ class DenseMLP(FeedForward):
         hn = h.tensor() if isinstance(h, LazyNorm) else h
         act = ctx.rows("dense_mlp.act", self.intermediate)
         self._product(ctx, act, hn, self.w_up, self.w_up_tiles)
-        ops.bias_act(act, act, self.up_bias, self.activation)
+        ops.bias_act(act, act, self.up_bias, self.activation, self.numbers)
         self._product(ctx, out, act, self.w_down, self.w_down_tiles)
 
     def forward_add(self, ctx, x, h):
+        if self.output_bias is None:        # the down product adds straight into the stream
+            hn = h.tensor() if isinstance(h, LazyNorm) else h
+            act = ctx.rows("dense_mlp.act", self.intermediate)
+            self._product(ctx, act, hn, self.w_up, self.w_up_tiles)
+            ops.bias_act(act, act, self.up_bias, self.activation, self.numbers)
+            n = act.shape[0]
+            if self.w_down_tiles is not None and n <= ops.SKINNY_MAX_ROWS:
+                ops.linear_fused(x, act, self.w_down_tiles, "add", **ctx.workspace.product_scratch(n, self.w_down_tiles))
+            else:
+                ops.linear(x, act, self.w_down, accumulate=True, **ctx.workspace.split_scratch(n, self.w_down))
+            return
         y = ctx.rows("mixer.rows_out", self.hidden, torch.float32)
         self.forward_into(ctx, y, h)
         if self.output_bias is not None:

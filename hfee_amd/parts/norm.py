@@ -1,7 +1,8 @@
 """RMSNorm (/root/reference/internal/ggml/ops.go:124-134): y = x / sqrt(mean(x^2) + eps) * w,
 the sum in float32, x the float32 residual stream, y in the engine's dtype (with the parameter
 `weight_offset` the stored weight lies around zero and the norm multiplies by offset + w: the sum
-is made once, in float32, when the weight is bound); and "none" for a
+is made once, in float32, when the weight is bound); "layernorm": y = (x - mean) / sqrt(variance + eps) * w
+with the variance as the mean of the squared deviations and no bias; and "none" for a
 place where a model has no norm (the rows as they are, in the engine's dtype)."""
 from __future__ import annotations
 
@@ -36,6 +37,26 @@ class RMSNorm(Norm):
 
     def forward(self, ctx, out, x, rows=None):
         ops.rmsnorm(out, x, self.weight, self.eps, rows)
+
+
+@register_norm("layernorm")
+class LayerNorm(Norm):
+    """The mean taken off, then the root mean square of what is left: not of the form that products
+    fold into their first or last step (no `fused_form`), so it always runs as a launch of its own."""
+    graph_safe = True
+
+    def __init__(self, spec: NormSpec, name: str):
+        self.width, self.eps, self.name = spec.width, spec.eps, name
+        self.weight = None
+
+    def tensor_specs(self):
+        return [TensorSpec(self.name, (self.width,), role="vector", init=("one_plus_normal",))]
+
+    def bind(self, tensors):
+        self.weight = tensors[self.name].contiguous()
+
+    def forward(self, ctx, out, x, rows=None):
+        ops.layernorm(out, x, self.weight, self.eps, rows)
 
 
 @register_norm("none")

@@ -1,0 +1,196 @@
+"""Mixers that keep a matrix of fixed size for every request instead of a growing cache.
+
+Both hold, for each head, S [dim, vdim] in float32 in the request's state slot (zero when the request
+is admitted), walk a step's tokens of a request in order from it, and leave the new state there; a
+decay acts on the rows of S, one number a key channel.  What enters the recurrence besides the
+projections themselves is made in float32: decays, step sizes, writing strengths, unit norms.
+
+"gated_delta": q, k (`num_qk_heads` heads of `dim`; head h reads q/k head h // (heads / qk heads)) and v
+(`num_heads` heads of `vdim`) each pass a short causal convolution per channel (`conv` taps, no bias,
+zeros before the sequence's start; the last conv - 1 inputs are state too) and a SiLU; q and k
+become unit vectors per head, x / sqrt(sum(x^2) + unit_eps), q also times dim^(-1/2);
+b = sigmoid(W_b h) a head; a = exp(-exp(A_h) softplus(W_a2 W_a1 h + dt_bias)) a head and key channel.
+Per token S <- diag(a) S; u = b (v - S^T k); S <- S + k u^T; o = S^T q.  Each head's o is divided by
+its root mean square (eps `norm_eps`), times a weight shared by the heads, times
+sigmoid(W_g2 W_g1 h); then the output product.
+
+"gla": q = W_q h dim^(-1/2), k, v; a = sigmoid(W_a2 W_a1 h + bias)^(1/tau);
+S <- diag(a) S + k v^T; o = S^T q; each head's o normed as above with a weight shared by the heads,
+the heads side by side times silu(W_g h); then the output product.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import MixerSpec
+from ..kernels import ops
+from ..weights.spec import TensorSpec
+from .base import LazyNorm, Mixer, register_mixer
+from .kv_attention import product, tiles_of
+
+
+class _StateMixer(Mixer):
+    graph_safe = True
+
+    def _names(self, spec, defaults):
+        given = dict(spec.get("names") or ())
+        return {role: self.prefix + given.get(role, default) for role, default in defaults.items()}
+
+    def cache_spec(self):
+        return None
+
+    def _segments(self, ctx):
+        return ctx.segment_rows, ctx.segment_lengths, ctx.segment_slots
+
+
+@register_mixer("gated_delta")
+class GatedDelta(_StateMixer):
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.heads = spec.get("num_heads")
+        self.qk_heads = spec.get("num_qk_heads", self.heads)
+        self.dim, self.vdim = spec.get("dim"), spec.get("vdim")
+        self.taps = spec.get("conv")
+        self.decay_rank, self.gate_rank = spec.get("decay_rank"), spec.get("gate_rank")
+        self.unit_eps = float(spec.get("unit_eps", 1e-6))
+        self.norm_eps = float(spec.get("norm_eps", 1e-6))
+        if self.heads % self.qk_heads:
+            raise ValueError(f"{self.heads} heads are not a multiple of {self.qk_heads} query/key heads")
+        if self.taps < 1:
+            raise ValueError("the short convolution has at least one tap")
+        self.names = self._names(spec, dict(
+            q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", q_conv="q_conv.weight", k_conv="k_conv.weight",
+            v_conv="v_conv.weight", b="b_proj.weight", a_log="A_log", norm="norm.weight", a_down="a_down.weight",
+            a_up="a_up.weight", dt_bias="dt_bias", g_down="g_down.weight", g_up="g_up.weight", o="o_proj.weight"))
+        self.qk_width, self.v_width = self.qk_heads * self.dim, self.heads * self.vdim
+        self.channels = 2 * self.qk_width + self.v_width
+
+    def tensor_specs(self):
+        n, H, D = self.names, self.heads, self.dim
+        specs = [TensorSpec(n["q"], (self.qk_width, self.hidden)), TensorSpec(n["q_conv"], (self.qk_width, self.taps), role="vector"),
+                 TensorSpec(n["k"], (self.qk_width, self.hidden)), TensorSpec(n["k_conv"], (self.qk_width, self.taps), role="vector"),
+                 TensorSpec(n["v"], (self.v_width, self.hidden)), TensorSpec(n["v_conv"], (self.v_width, self.taps), role="vector"),
+                 TensorSpec(n["b"], (H, self.hidden)), TensorSpec(n["a_log"], (H,), role="vector"),
+                 TensorSpec(n["norm"], (self.vdim,), role="vector", init=("one_plus_normal",)),
+                 TensorSpec(n["a_down"], (self.decay_rank, self.hidden)), TensorSpec(n["a_up"], (H * D, self.decay_rank)),
+                 TensorSpec(n["dt_bias"], (H * D,), role="vector"),
+                 TensorSpec(n["g_down"], (self.gate_rank, self.hidden)), TensorSpec(n["g_up"], (self.v_width, self.gate_rank)),
+                 TensorSpec(n["o"], (self.hidden, self.v_width))]
+        return specs
+
+    def bind(self, tensors):
+        n = self.names
+        f32 = lambda name: tensors.pop(name).to(torch.float32).contiguous()      # noqa: E731
+        # one product for everything that reads the layer's input: [q | k | v | a_down | g_down | b]
+        self.w_in = torch.cat([tensors.pop(n[r]) for r in ("q", "k", "v", "a_down", "g_down", "b")], dim=0).contiguous()
+        self.at_a = self.channels
+        self.at_g = self.at_a + self.decay_rank
+        self.at_b = self.at_g + self.gate_rank
+        self.conv_taps = torch.cat([f32(n["q_conv"]), f32(n["k_conv"]), f32(n["v_conv"])], dim=0).contiguous()
+        self.a_log, self.dt_bias, self.norm_weight = f32(n["a_log"]), f32(n["dt_bias"]), f32(n["norm"])
+        self.w_a_up, self.w_g_up = tensors.pop(n["a_up"]).contiguous(), tensors.pop(n["g_up"]).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.w_in_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_in, self.w_o)
+        self.w_a_up_tiles, self.w_g_up_tiles = tiles_of(self.dtype, self.w_a_up, self.w_g_up)
+
+    def state_specs(self):
+        return [(self.prefix + "state", (self.heads, self.dim, self.vdim), torch.float32),
+                (self.prefix + "conv_state", (self.taps - 1, self.channels), self.dtype)]
+
+    def prepare(self, info):
+        self.state = info.storage.states[self.prefix + "state"]
+        self.conv_state = info.storage.states[self.prefix + "conv_state"]
+
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        H, G, D, V = self.heads, self.qk_heads, self.dim, self.vdim
+        rows, lengths, slots = self._segments(ctx)
+        total = self.w_in.shape[0]       # (rows of a multiple of 8 elements, so that blocks of columns stay aligned)
+        proj = ctx.rows("gated_delta.in", (total + 7) // 8 * 8)[:, :total]
+        product(ctx, proj, hn, self.w_in, self.w_in_tiles)
+        raw = proj[:, :self.channels]
+        y = ctx.rows("gated_delta.conv", self.channels, torch.float32)
+        ops.short_conv_silu(y, raw, self.conv_state, self.conv_taps, ctx.token_segment, rows, slots)
+        ops.short_conv_keep(self.conv_state, raw, rows, lengths, slots)
+        q, k, v = y[:, :self.qk_width], y[:, self.qk_width:2 * self.qk_width], y[:, 2 * self.qk_width:]
+        ops.unit_heads(q, G, D, self.unit_eps, D ** -0.5)
+        ops.unit_heads(k, G, D, self.unit_eps, 1.0)
+        step = ctx.rows("gated_delta.step", H * D)
+        product(ctx, step, proj[:, self.at_a:self.at_g], self.w_a_up, self.w_a_up_tiles)
+        decay = ctx.rows("gated_delta.decay", H * D, torch.float32)
+        ops.scan_gate(decay, step, "step_decay", bias=self.dt_bias, per_head=self.a_log, head_width=D)
+        beta = ctx.rows("gated_delta.beta", H, torch.float32)
+        ops.scan_gate(beta, proj[:, self.at_b:self.at_b + H], "sigmoid")
+        o = ctx.rows("gated_delta.read", self.v_width, torch.float32)
+        ops.linear_scan(o, self.state, q, k, v, decay, beta, rows, lengths, slots, H, G, D, V, "delta")
+        gate = ctx.rows("gated_delta.gate", self.v_width)
+        product(ctx, gate, proj[:, self.at_g:self.at_b], self.w_g_up, self.w_g_up_tiles)
+        gated = ctx.rows("gated_delta.out", self.v_width)
+        ops.head_norm_gate(gated, o, gate, self.norm_weight, H, V, self.norm_eps, "sigmoid")
+        product(ctx, x, gated, self.w_o, self.w_o_tiles, add=True)
+
+
+@register_mixer("gla")
+class GatedLinearAttention(_StateMixer):
+    def __init__(self, spec: MixerSpec, prefix: str, dtype: torch.dtype):
+        self.prefix, self.dtype = prefix, dtype
+        self.hidden = spec.get("hidden")
+        self.heads = spec.get("num_heads")
+        self.dim, self.vdim = spec.get("dim"), spec.get("vdim")
+        self.tau = float(spec.get("tau"))
+        self.decay_rank = spec.get("decay_rank")
+        self.norm_eps = float(spec.get("norm_eps", 1e-6))
+        if self.tau <= 0:
+            raise ValueError("tau must be positive")
+        self.names = self._names(spec, dict(
+            q="q_proj.weight", k="k_proj.weight", v="v_proj.weight", g="g_proj.weight", o="o_proj.weight",
+            norm="norm.weight", a_down="a_down.weight", a_up="a_up.weight", a_bias="a_up.bias"))
+        self.qk_width, self.v_width = self.heads * self.dim, self.heads * self.vdim
+
+    def tensor_specs(self):
+        n = self.names
+        return [TensorSpec(n["q"], (self.qk_width, self.hidden)), TensorSpec(n["k"], (self.qk_width, self.hidden)),
+                TensorSpec(n["v"], (self.v_width, self.hidden)), TensorSpec(n["g"], (self.v_width, self.hidden)),
+                TensorSpec(n["o"], (self.hidden, self.v_width)),
+                TensorSpec(n["norm"], (self.vdim,), role="vector", init=("one_plus_normal",)),
+                TensorSpec(n["a_down"], (self.decay_rank, self.hidden)), TensorSpec(n["a_up"], (self.qk_width, self.decay_rank)),
+                TensorSpec(n["a_bias"], (self.qk_width,), role="vector")]
+
+    def bind(self, tensors):
+        n = self.names
+        # one product for everything that reads the layer's input: [q | k | v | g | a_down]
+        self.w_in = torch.cat([tensors.pop(n[r]) for r in ("q", "k", "v", "g", "a_down")], dim=0).contiguous()
+        self.at_g = 2 * self.qk_width + self.v_width
+        self.at_a = self.at_g + self.v_width
+        self.w_a_up = tensors.pop(n["a_up"]).contiguous()
+        self.a_bias = tensors.pop(n["a_bias"]).to(torch.float32).contiguous()
+        self.norm_weight = tensors.pop(n["norm"]).to(torch.float32).contiguous()
+        self.w_o = tensors.pop(n["o"]).contiguous()
+        self.w_in_tiles, self.w_o_tiles, self.w_a_up_tiles = tiles_of(self.dtype, self.w_in, self.w_o, self.w_a_up)
+
+    def state_specs(self):
+        return [(self.prefix + "state", (self.heads, self.dim, self.vdim), torch.float32)]
+
+    def prepare(self, info):
+        self.state = info.storage.states[self.prefix + "state"]
+
+    def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
+        hn = h.tensor() if isinstance(h, LazyNorm) else h
+        H, D, V = self.heads, self.dim, self.vdim
+        rows, lengths, slots = self._segments(ctx)
+        total = self.w_in.shape[0]
+        proj = ctx.rows("gla.in", (total + 7) // 8 * 8)[:, :total]
+        product(ctx, proj, hn, self.w_in, self.w_in_tiles)
+        qkv = ctx.rows("gla.qkv", self.at_g, torch.float32)
+        ops.scan_gate(qkv, proj[:, :self.at_g], "cast", number=D ** -0.5, first_columns=self.qk_width)
+        q, k, v = qkv[:, :self.qk_width], qkv[:, self.qk_width:2 * self.qk_width], qkv[:, 2 * self.qk_width:]
+        z = ctx.rows("gla.z", self.qk_width)
+        product(ctx, z, proj[:, self.at_a:], self.w_a_up, self.w_a_up_tiles)
+        decay = ctx.rows("gla.decay", self.qk_width, torch.float32)
+        ops.scan_gate(decay, z, "root_sigmoid", bias=self.a_bias, number=self.tau)
+        o = ctx.rows("gla.read", self.v_width, torch.float32)
+        ops.linear_scan(o, self.state, q, k, v, decay, None, rows, lengths, slots, H, H, D, V, "decay_add")
+        gated = ctx.rows("gla.out", self.v_width)
+        ops.head_norm_gate(gated, o, proj[:, self.at_g:self.at_a], self.norm_weight, H, V, self.norm_eps, "silu")
+        product(ctx, x, gated, self.w_o, self.w_o_tiles, add=True)

@@ -193,7 +193,9 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int,
                     help="most tokens that live requests hold at any time (the cache pool is made for it)")
     ap.add_argument("--page-size", type=int, default=16)
-    ap.add_argument("--max-requests", type=int, default=64, help="most requests that are live at a time")
+    ap.add_argument("--max-requests", type=int, default=4,
+                    help="most requests that are live at a time: the engine has this many state slots, used again "
+                    "as requests end")
     ap.add_argument("--random-weights", action="store_true",
                     help="read config.json only; the weights are seeded random ones")
     ap.add_argument("--seed", type=int, default=0, help="seed of the random weights")

@@ -23,7 +23,8 @@ from .spec import TensorSpec
 def random_tensor(spec: TensorSpec, seed: int, std: float, dtype: torch.dtype,
                   device="cpu") -> torch.Tensor:
     """The tensor that `spec` declares: init ("normal",) is N(0, std), ("one_plus_normal",)
-    1 + N(0, std), ("zeros",), ("randint", bound) int32 in [0, bound).  Float64 rounded once to
+    1 + N(0, std), ("zeros",), ("randint", bound) int32 in [0, bound), ("distinct_in_row", bound) the same
+    with no two alike in a row of a 2-D tensor.  Float64 rounded once to
     float32, then to `dtype`; the same numbers on the CPU and on the GPU."""
     kind = spec.init[0]
     key = random_stream.tensor_key(seed, spec.name)
@@ -33,6 +34,15 @@ def random_tensor(spec: TensorSpec, seed: int, std: float, dtype: torch.dtype,
         count *= n
     if kind == "zeros":
         return torch.zeros(shape, dtype=dtype, device=device)
+    if kind == "distinct_in_row":
+        # [rows, columns] of integers below a bound, no two alike in a row: a random first column,
+        # the others count on from it
+        rows, columns = shape
+        bound = spec.init[1]
+        if columns > bound:
+            raise ValueError(f"tensor {spec.name}: {columns} different integers below {bound} do not exist")
+        first = random_tensor(TensorSpec(spec.name, (rows,), spec.role, ("randint", bound)), seed, std, dtype, device)
+        return ((first.to(torch.int64)[:, None] + torch.arange(columns, device=first.device)[None, :]) % bound).to(torch.int32)
     if kind not in ("normal", "one_plus_normal", "randint"):
         raise ValueError(f"tensor {spec.name}: unknown init {spec.init!r}")
     if torch.device(device).type == "cpu":

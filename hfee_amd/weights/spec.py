@@ -12,5 +12,5 @@ class TensorSpec:
                           # "vector": cast likewise unless stored in 32-bit (then kept);
                           # "table": integers, kept as int32
     init: tuple = ("normal",)   # random-weights mode: ("normal",) | ("one_plus_normal",) |
-                                # ("zeros",) | ("randint", high)
+                                # ("zeros",) | ("randint", high) | ("distinct_in_row", high)
     optional: bool = False
