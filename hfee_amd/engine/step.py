@@ -287,7 +287,7 @@ class Engine:
                 bt[i, :len(t)] = t          # blocks that a window has given back hold 0 and are never read
             plan.add(f"block_tables.{g}", bt)
         if decode_only:
-            plan.host["graph.max_context"] = max(widths) * self.page_size
+            plan.host["graph.max_context"] = max(widths, default=0) * self.page_size
         self.model.plan(plan)
         plan.n, plan.wanted, plan.max_position = n, len(logit_rows), int(positions.max())
         plan.graph_key = None

@@ -1,0 +1,100 @@
+"""The Sabezen configuration and the plain implementation, without a GPU: what config.json gives and
+what it leaves to the tensors' shapes, the tensors that the parts declare, and properties that the
+plain implementation must have by the design's definition (a prefix's logits do not change with
+what follows; an attention layer sees nothing before its chunk; a recurrent layer does)."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+import plain_sabezen as ps
+import sabezen_util as su
+
+
+def test_the_configuration_reads_ranks_from_the_tensors(tmp_path):
+    from hfee_amd.config import ConfigError, config_from_dict, config_from_folder
+    folder = su.make_folder(tmp_path / "a", su.S_A, seed=1)
+    with open(f"{folder}/config.json") as f:
+        assert "decay_rank" not in json.dumps(json.load(f))
+    cfg = config_from_folder(folder)
+    assert cfg.layers[1].mixer.decay_rank == 8 and cfg.layers[1].mixer.gate_rank == 8 and cfg.layers[2].mixer.decay_rank == 8
+    assert cfg.embedding_scale == 3.0 and cfg.layers[0].mixer.chunk == 24 and cfg.layers[2].mlp is None
+    assert cfg.layers[1].mlp.top == 2 and cfg.layers[1].mlp.experts == 5
+    again = config_from_dict(cfg.to_dict())
+    assert again == cfg
+    stripped = json.loads(json.dumps(su.S_A))
+    stripped["layers"][1]["mixer"].pop("decay_rank")
+    with pytest.raises(ConfigError, match="ranks"):
+        config_from_dict(stripped)
+    bad = json.loads(json.dumps(su.S_A))
+    bad["layers"][0]["mixer"]["vdim"] = 8
+    with pytest.raises(ConfigError, match="vdim"):
+        config_from_dict(bad)
+    bad = json.loads(json.dumps(su.S_A))
+    bad["layers"][3]["mlp"]["router"]["top"] = 9
+    with pytest.raises(ConfigError, match="experts"):
+        config_from_dict(bad)
+    bad = json.loads(json.dumps(su.S_A))
+    bad["layers"][2]["type"] = "window"
+    with pytest.raises(ConfigError, match="unknown mixer"):
+        config_from_dict(bad)
+
+
+def test_the_parts_declare_the_design_s_tensors():
+    from hfee_amd.config import config_from_dict
+    from hfee_amd.engine.model import declared_tensors
+    specs = {s.name: tuple(s.shape) for s in declared_tensors(config_from_dict(su.S_A))}
+    assert specs["embed"] == (131, 64) and specs["head"] == (131, 64) and specs["final.norm"] == (64,)
+    assert specs["l0.mix.q"] == (64, 64) and specs["l0.mix.k"] == (32, 64) and specs["l0.mix.talk"] == (4, 4)
+    assert "l0.mix.v" not in specs and specs["l0.mlp.act"] == (2,)
+    assert specs["l1.mix.q.conv"] == (16, 4) and specs["l1.mix.v.conv"] == (64, 4) and specs["l1.mix.b"] == (4, 64)
+    assert specs["l1.mix.a2"] == (32, 8) and specs["l1.mix.g2"] == (64, 8) and specs["l1.mix.dt_bias"] == (32,)
+    assert specs["l1.mlp.table"] == (131, 2) and specs["l1.mlp.e4.down"] == (64, 24) and "l1.mlp.e5.up" not in specs
+    assert specs["l2.mix.a2.b"] == (32,) and specs["l2.mix.g"] == (16, 64) and not any(n.startswith("l2.mlp") for n in specs)
+    table = su.make_tensors(su.S_A, 5)["l1.mlp.table"]
+    assert table.dtype == torch.int32 and int(table.min()) >= 0 and int(table.max()) < 5
+    assert bool((table[:, 0] != table[:, 1]).all())
+
+
+def _logits(cj, w, tokens):
+    return ps.forward(cj, w, tokens, dtype=torch.float64).numpy()
+
+
+def test_a_prefix_does_not_depend_on_what_follows():
+    w = su.make_tensors(su.S_A, 3)
+    toks = np.random.default_rng(0).integers(0, 131, size=60).tolist()
+    whole = _logits(su.S_A, w, toks)
+    assert np.abs(_logits(su.S_A, w, toks[:33]) - whole[:33]).max() < 1e-9
+
+
+def test_what_an_attention_layer_and_a_recurrent_layer_see():
+    """A model of one attention layer forgets everything at a chunk's edge; a recurrent one does not."""
+    toks = np.random.default_rng(1).integers(0, 50, size=25).tolist()
+    other = [(toks[0] + 1) % 50] + toks[1:]
+    cj, w = su.SINGLE["attention"], su.make_tensors(su.SINGLE["attention"], 2)      # chunks of 10
+    a, b = _logits(cj, w, toks), _logits(cj, w, other)
+    assert np.abs(a[1:10] - b[1:10]).max() > 1e-4            # same chunk: seen
+    assert np.abs(a[10:] - b[10:]).max() < 1e-12             # behind the edge: not seen
+    for name in ("delta", "gla"):
+        cj, w = su.SINGLE[name], su.make_tensors(su.SINGLE[name], 2)
+        a, b = _logits(cj, w, toks), _logits(cj, w, other)
+        assert np.abs(a[24] - b[24]).max() > 1e-6
+
+
+def test_the_sink_takes_its_share():
+    """With scores far below zero nearly all of the softmax's weight goes to the sink, which has no value:
+    the attention's output shrinks towards nothing."""
+    g = torch.Generator().manual_seed(0)
+    H, D, T = 2, 4, 6
+    m = {"heads": H, "kv_heads": H, "dim": D, "scale": 1.0, "mask": {"size": 100}, "rot": {"dims": 0, "base": 10.0}}
+    w = {"m.q": torch.eye(2 * H * D)[:H * D].double(), "m.k": torch.eye(2 * H * D)[H * D:].double(),
+         "m.talk": torch.eye(H).double(), "m.o": torch.eye(H * D).double()}
+    k = torch.randn(T, H * D, generator=g).double()
+    towards = ps.chunked_talking_attention(torch.cat([k, k], dim=1), w, "m.", m, 1e-6)
+    away = ps.chunked_talking_attention(torch.cat([-k, k], dim=1), w, "m.", m, 1e-6)
+    w["m.talk"] = torch.eye(H).double() * 6
+    far_away = ps.chunked_talking_attention(torch.cat([-k, k], dim=1), w, "m.", m, 1e-6)
+    # the first token sees its own key only: its weight is e^s / (1 + e^s)
+    assert float(far_away[0].abs().max()) < float(away[0].abs().max()) < float(towards[0].abs().max())
+    assert float(far_away[0].abs().max()) < 1e-9 and float(towards[0].abs().max()) > 0.9 * float(k[0].abs().max())
