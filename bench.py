@@ -58,6 +58,15 @@ VOFEZEN_SIZES = {
     "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, q_rank=1536),
 }
 
+# The Sabezen design at the same two layer sizes: its layers go round attention over chunks of 1,024
+# keys (heads and head size of the Llama layer beside it), the gated delta rule and gated linear
+# attention (heads of 128 key and 256 value channels, as many as make the values as wide as the
+# model), with a dense feed-forward of two matrices and sixteen experts (two a token) in turn.
+SABEZEN_SIZES = {
+    "2048-wide": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=12288, llama_ff=8192, expert_ff=1024),
+    "4096-wide": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=21504, llama_ff=14336, expert_ff=2048),
+}
+
 
 CONTEXT = 8192
 PROMPT = 1024
@@ -100,6 +109,15 @@ def parse(argv=None):
                     help="with --vofezen: only this layer size")
     ap.add_argument("--vofezen-design", choices=["both", "vofezen", "llama"], default="both",
                     help="with --vofezen: only one of the two designs (for profiling)")
+    ap.add_argument("--sabezen", action="store_true",
+                    help="instead of the default run: the Sabezen design (parallel blocks; attention over chunks with "
+                         "mixed heads, the gated delta rule and gated linear attention over per-request states; dense "
+                         "and table-routed expert feed-forwards) at two layer sizes beside the Llama decoder at equal "
+                         "width and heads; prints its own line")
+    ap.add_argument("--sabezen-size", choices=sorted(SABEZEN_SIZES), default=None,
+                    help="with --sabezen: only this layer size")
+    ap.add_argument("--sabezen-design", choices=["both", "sabezen", "llama"], default="both",
+                    help="with --sabezen: only one of the two designs (for profiling)")
     ap.add_argument("--no-extra-points", action="store_true",
                     help="skip the other shapes and the longer context that the default run adds under `points`")
     return ap.parse_args(argv)
@@ -189,11 +207,31 @@ def vofezen_configs(size: dict, layers: int, vocab: int = 32000):
     return vof, llama
 
 
+def sabezen_configs(size: dict, layers: int, vocab: int = 32000):
+    """(config.json keys of the Sabezen model, of the Llama model beside it)."""
+    d, H, G, hd = size["width"], size["heads"], size["kv_heads"], size["dim"]
+    att = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                                          "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": hd // 2}}}
+    heads = d // 256
+    dlt = {"type": "channel_delta", "mixer": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 256, "conv": 4,
+                                              "decay_rank": 64, "gate_rank": 128}}
+    gla = {"type": "gla", "mixer": {"heads": heads, "dim": 128, "vdim": 256, "tau": 16.0, "decay_rank": 16}}
+    dense = {"kind": "dense", "ff": size["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": size["expert_ff"]}, "router": {"experts": 16, "top": 2}}
+    sab = {"architecture": "Sabezen", "vocab": vocab, "width": d, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+           "layers": [dict((att, dlt, gla)[i % 3], mlp=(dense, moe)[i % 2]) for i in range(layers)]}
+    llama = dict(BASE_8B, architectures=["LlamaForCausalLM"], num_hidden_layers=layers, hidden_size=d,
+                 num_attention_heads=H, num_key_value_heads=G, head_dim=hd, intermediate_size=size["llama_ff"],
+                 vocab_size=vocab)
+    return sab, llama
+
+
 def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     """Prefill of 2,048 tokens and decode at `batch` requests of 1,024-token prompts for any
     registered architecture: times, and the fractions of the HBM and matrix peaks by the bytes a
     step must read (every matrix once, the cache of the live requests) and the flops of the
     products and of the attention as the kernels run it."""
+    import numpy as np
     import torch
 
     from hfee_amd.cache import bytes_per_token
@@ -203,12 +241,30 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
     cfg = config_from_dict(cj)
     model = random_model(cfg, seed=0, dtype="bfloat16", device="cuda:0", std=0.02)
     spec = model.spec
-    matrices = [t for t in model.tensor_specs() if len(t.shape) == 2 and t.name != spec.embedding_name]
-    weight_bytes = 2 * sum(t.shape[0] * t.shape[1] for t in matrices)
-    layer_flops_a_token = 2 * sum(t.shape[0] * t.shape[1] for t in matrices)
+    matrices = [t for t in model.tensor_specs() if len(t.shape) == 2 and t.name != spec.embedding_name and t.role == "matrix"]
+    # (experts: a token multiplies by `top` of them; a decode step reads at most batch * top of them)
+    used, read = {}, {}
+    for ls in spec.layers:
+        f = ls.feed_forward
+        if f is not None and f.kind == "table_moe":
+            used[ls.name_of("feed_forward", "")] = f.get("top") / f.get("experts")
+            read[ls.name_of("feed_forward", "")] = min(1.0, batch * f.get("top") / f.get("experts"))
+
+    def share(t, table):
+        return next((v for k, v in table.items() if t.name.startswith(k)), 1.0)
+    weight_bytes = 2 * sum(t.shape[0] * t.shape[1] * share(t, read) for t in matrices)
+    layer_flops_a_token = 2 * sum(t.shape[0] * t.shape[1] * share(t, used) for t in matrices)
     attention_dims = 0          # (key size + value size) x heads, summed over the layers, as the kernels see them
+    chunked_flops = 0.0         # attention over chunks: the keys that a prompt of PREFILL tokens sees
+    state_bytes = sum(4 * int(np.prod(shape)) for _, shape, dt in model.state_specs() if dt == torch.float32)
+    scan_flops_a_token = 0      # the recurrences' multiply-adds on the vector units, counted apart
     for ls in spec.layers:
         m = ls.mixer
+        if m.kind == "mixed_attention":
+            seen = sum(i % m.get("chunk") + 1 for i in range(PREFILL)) if m.get("chunk") else PREFILL * (PREFILL + 1) / 2
+            chunked_flops += 2.0 * 2 * m.get("dim") * m.get("num_heads") * seen
+        elif m.kind in ("gated_delta", "gla"):
+            scan_flops_a_token += 2 * (4 if m.kind == "gated_delta" else 3) * m.get("num_heads") * m.get("dim") * m.get("vdim")
         if m.kind == "attention":
             attention_dims += 2 * m.get("head_dim") * m.get("num_heads")
         elif m.kind == "kv_attention":
@@ -231,7 +287,7 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
         dt = time.perf_counter() - t
         engine.release(("prefill", i))
         best = dt if best is None else min(best, dt)
-    prefill_flops = PREFILL * layer_flops_a_token + 2.0 * attention_dims * PREFILL * (PREFILL + 1) / 2
+    prefill_flops = PREFILL * layer_flops_a_token + 2.0 * attention_dims * PREFILL * (PREFILL + 1) / 2 + chunked_flops
     sched = Scheduler(engine, sampler, max_num_seqs=batch, max_batch_tokens=PREFILL, num_ctx=context)
     params = SamplingParams.greedy(num_predict=-1, ignore_eos=True)
     for i in range(batch):
@@ -246,7 +302,12 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
         sched.step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t) / steps
-    step_bytes = weight_bytes + batch * (PROMPT + warmup + steps / 2) * bytes_per_token(engine.groups, torch.bfloat16)
+    # (a layer of attention over chunks reads its chunk only; the states are read and written)
+    context_read = PROMPT + warmup + steps / 2
+    chunks = [ls.mixer.get("chunk") for ls in spec.layers if ls.mixer.kind == "mixed_attention" and ls.mixer.get("chunk")]
+    if chunks:
+        context_read = context_read % min(chunks) + 1
+    step_bytes = weight_bytes + batch * context_read * bytes_per_token(engine.groups, torch.bfloat16) + 2 * batch * state_bytes
     for r in list(sched.running):
         sched.cancel(r.request_id)
     while sched.has_work():
@@ -256,6 +317,9 @@ def design_point(cj: dict, batch: int, steps: int, warmup: int) -> dict:
            f"decode_b{batch}_tok_s": round(batch / dt, 1), f"decode_b{batch}_ms_per_step": round(dt * 1e3, 4),
            "decode_frac_of_hbm_peak": round(step_bytes / dt / HBM_PEAK, 4),
            "weight_gb": round(weight_bytes / 1e9, 3), "graph_replays": engine.graph_replays}
+    if state_bytes:
+        out["state_mb_a_request"] = round(state_bytes / 1e6, 3)
+        out["scan_gflop_a_prefill"] = round(PREFILL * scan_flops_a_token / 1e9, 2)
     del sched, sampler, engine, model
     torch.cuda.empty_cache()
     return out
@@ -279,11 +343,32 @@ def vofezen_compare(args) -> dict:
             "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": layers, "points": points}
 
 
+def sabezen_compare(args) -> dict:
+    import hfee_amd  # noqa: F401
+    layers = args.layers or 6
+    points = {}
+    for name, size in SABEZEN_SIZES.items():
+        if args.sabezen_size not in (None, name):
+            continue
+        sab, llama = sabezen_configs(size, layers)
+        for design, cj in (("sabezen", sab), ("llama", llama)):
+            if args.sabezen_design not in ("both", design):
+                continue
+            print(f"[bench] {design} {name}, {layers} layers", file=sys.stderr, flush=True)
+            points[f"{design}_{name}"] = design_point(cj, args.batch, min(args.steps, 32), min(args.warmup, 4))
+    return {"metric": "Sabezen beside Llama at equal layer sizes: prefill of 2,048 tokens, decode at batch %d and "
+                      "1,024-token prompts (bf16, random weights)" % args.batch,
+            "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16", "layers": layers, "points": points}
+
+
 def main(argv=None) -> int:
     args = parse(argv)
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.sabezen:
+        print(json.dumps(sabezen_compare(args)), flush=True)
+        return 0
     if args.vofezen:
         print(json.dumps(vofezen_compare(args)), flush=True)
         return 0

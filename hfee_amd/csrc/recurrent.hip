@@ -10,8 +10,9 @@
 // `linear_scan` walks the tokens that a step brings for a request one after the other, from the
 // state that the steps before left in the request's slot, and leaves the new state there: a
 // portion of a prompt and a single token are the same kernel, and a token's result does not
-// depend on where its prompt was cut.  A thread owns D/4 rows of one column of S; four lanes
-// share a column and add their parts up in a fixed order.
+// depend on where its prompt was cut.  A wave owns four columns of S, a lane every sixteenth row of one
+// of them; the sixteen lanes of a column add their parts up in a fixed order.  In memory the state of a
+// head lies as [blocks of four columns][D][4] (values that are no multiple of four are filled up).
 //
 // Around it, each in float32 whatever the engine's dtype:
 //   short_conv_silu     y_t = silu(sum_j taps[K-1-j] x_(t-j)) per channel, the K-1 inputs before the
@@ -100,7 +101,47 @@ __global__ __launch_bounds__(256) void scan_gate_kernel(float* __restrict__ out,
   out[t * ldo + c] = r;
 }
 
-// grid (column blocks of 16, heads, segments), 64 threads: lane = 16 (part of D) + column.
+// grid (column blocks of 4, heads, segments), one wave: lane = 16 * column + part.  A lane owns the rows
+// d = 16 i + part (i < DPT) of its column of S, so that the sixteen lanes of a column hold sixteen
+// neighbouring rows and a load instruction of the wave covers 64 neighbouring floats of the state, which
+// lies in memory as [slot][head][column block][D][4].  The rows' products are added in two chains a
+// lane and then over the sixteen lanes of the column in a fixed tree.  What the next token needs is asked
+// for before the current one is worked on.
+constexpr int kScanParts = 16, kScanColumns = 4;
+
+template <int DPT>
+struct ScanInputs {
+  float k[DPT], q[DPT], a[DPT], v, b;
+};
+
+template <int DPT, int RULE>
+__device__ __forceinline__ void scan_load(ScanInputs<DPT>& in, const float* __restrict__ q, int64_t ldq,
+                                          const float* __restrict__ k, int64_t ldk, const float* __restrict__ v, int64_t ldv,
+                                          const float* __restrict__ decay, int64_t ldd, const float* __restrict__ beta,
+                                          int64_t ldb, int t, int g, int h, int col, bool live, int part, int D, int V) {
+  const float* qt = q + (int64_t)t * ldq + (int64_t)g * D;
+  const float* kt = k + (int64_t)t * ldk + (int64_t)g * D;
+  const float* at = decay + (int64_t)t * ldd + (int64_t)h * D;
+#pragma unroll
+  for (int i = 0; i < DPT; ++i) {
+    const int d = i * kScanParts + part;
+    const bool in_d = d < D;
+    in.k[i] = in_d ? kt[d] : 0.f;
+    in.q[i] = in_d ? qt[d] : 0.f;
+    in.a[i] = in_d ? at[d] : 0.f;
+  }
+  in.v = live ? v[(int64_t)t * ldv + (int64_t)h * V + col] : 0.f;
+  in.b = RULE == 1 ? beta[(int64_t)t * ldb + h] : 1.f;
+}
+
+__device__ __forceinline__ float column_sum(float x) {      // over the sixteen lanes of a column
+  x += __shfl_xor(x, 1, kWave);
+  x += __shfl_xor(x, 2, kWave);
+  x += __shfl_xor(x, 4, kWave);
+  x += __shfl_xor(x, 8, kWave);
+  return x;
+}
+
 template <int DPT, int RULE>
 __global__ __launch_bounds__(64) void linear_scan_kernel(
     float* __restrict__ out, int64_t ldo, float* __restrict__ state, const float* __restrict__ q, int64_t ldq,
@@ -108,55 +149,49 @@ __global__ __launch_bounds__(64) void linear_scan_kernel(
     int64_t ldd, const float* __restrict__ beta, int64_t ldb, const int* __restrict__ segment_rows,
     const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int heads, int qk_heads, int D, int V) {
   const int seg = blockIdx.z, h = blockIdx.y;
-  const int col = blockIdx.x * 16 + (threadIdx.x & 15), part = threadIdx.x >> 4;
+  const int part = threadIdx.x & (kScanParts - 1), c = threadIdx.x >> 4;
+  const int col = blockIdx.x * kScanColumns + c;
   const bool live = col < V;
-  const int d0 = part * DPT;
   const int g = h / (heads / qk_heads);
-  float* S = state + (((int64_t)segment_slots[seg] * heads + h) * D) * V + (live ? col : 0);
+  const int blocks = (V + kScanColumns - 1) / kScanColumns;
+  float* S = state + ((((int64_t)segment_slots[seg] * heads + h) * blocks + blockIdx.x) * D) * kScanColumns + c;
   float s[DPT];
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) s[i] = live && d0 + i < D ? S[(int64_t)(d0 + i) * V] : 0.f;
+  for (int i = 0; i < DPT; ++i) {
+    const int d = i * kScanParts + part;
+    s[i] = d < D ? S[(int64_t)d * kScanColumns] : 0.f;
+  }
   const int row0 = segment_rows[seg], len = segment_lengths[seg];
+  ScanInputs<DPT> now, next;
+  scan_load<DPT, RULE>(now, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, row0, g, h, col, live, part, D, V);
   for (int t = row0; t < row0 + len; ++t) {
-    const float* qt = q + (int64_t)t * ldq + (int64_t)g * D + d0;
-    const float* kt = k + (int64_t)t * ldk + (int64_t)g * D + d0;
-    const float* at = decay + (int64_t)t * ldd + (int64_t)h * D + d0;
-    float kk[DPT], qq[DPT], aa[DPT];
-#pragma unroll
-    for (int i = 0; i < DPT; ++i) {
-      const bool in = d0 + i < D;
-      kk[i] = in ? kt[i] : 0.f;
-      qq[i] = in ? qt[i] : 0.f;
-      aa[i] = in ? at[i] : 0.f;
-    }
-    const float vt = live ? v[(int64_t)t * ldv + (int64_t)h * V + col] : 0.f;
-    float u = vt;
+    if (t + 1 < row0 + len)
+      scan_load<DPT, RULE>(next, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, t + 1, g, h, col, live, part, D, V);
+    float u = now.v;
     if constexpr (RULE == 1) {
-      float dot = 0.f;
+      float d0 = 0.f, d1 = 0.f;
 #pragma unroll
       for (int i = 0; i < DPT; ++i) {
-        s[i] *= aa[i];
-        dot = fmaf(s[i], kk[i], dot);
+        s[i] *= now.a[i];
+        if (i & 1) d1 = fmaf(s[i], now.k[i], d1); else d0 = fmaf(s[i], now.k[i], d0);
       }
-      dot += __shfl_xor(dot, 16, kWave);
-      dot += __shfl_xor(dot, 32, kWave);
-      u = beta[(int64_t)t * ldb + h] * (vt - dot);
+      u = now.b * (now.v - column_sum(d0 + d1));
     }
-    float o = 0.f;
+    float o0 = 0.f, o1 = 0.f;
 #pragma unroll
     for (int i = 0; i < DPT; ++i) {
-      if constexpr (RULE == 1) s[i] = fmaf(kk[i], u, s[i]);
-      else s[i] = fmaf(s[i], aa[i], kk[i] * u);
-      o = fmaf(s[i], qq[i], o);
+      if constexpr (RULE == 1) s[i] = fmaf(now.k[i], u, s[i]);
+      else s[i] = fmaf(s[i], now.a[i], now.k[i] * u);
+      if (i & 1) o1 = fmaf(s[i], now.q[i], o1); else o0 = fmaf(s[i], now.q[i], o0);
     }
-    o += __shfl_xor(o, 16, kWave);
-    o += __shfl_xor(o, 32, kWave);
+    const float o = column_sum(o0 + o1);
     if (live && part == 0) out[(int64_t)t * ldo + (int64_t)h * V + col] = o;
+    now = next;
   }
-  if (live) {
 #pragma unroll
-    for (int i = 0; i < DPT; ++i)
-      if (d0 + i < D) S[(int64_t)(d0 + i) * V] = s[i];
+  for (int i = 0; i < DPT; ++i) {
+    const int d = i * kScanParts + part;
+    if (d < D) S[(int64_t)d * kScanColumns] = s[i];
   }
 }
 
@@ -263,14 +298,15 @@ HFEE_API int hfee_linear_scan(float* out, int64_t ldo, float* state, const float
   HFEE_REQUIRE(rule == 0 || (rule == 1 && beta != nullptr), "linear_scan: rule 0, or rule 1 with its writing strengths");
   HFEE_REQUIRE(ldq >= (int64_t)qk_heads * dim && ldk >= (int64_t)qk_heads * dim && ldv >= (int64_t)heads * vdim &&
                ldd >= (int64_t)heads * dim && ldo >= (int64_t)heads * vdim, "linear_scan: rows too short");
-  dim3 grid((vdim + 15) / 16, heads, segments);
-  const int per = (dim + 3) / 4;
+  dim3 grid((vdim + kScanColumns - 1) / kScanColumns, heads, segments);
+  HFEE_REQUIRE(grid.x <= 65535u * 32u, "linear_scan: values too wide");
+  const int per = (dim + kScanParts - 1) / kScanParts;
 #define LAUNCH(DPT, RULE)                                                                                             \
   linear_scan_kernel<DPT, RULE><<<grid, 64, 0, stream>>>(out, ldo, state, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, \
       segment_rows, segment_lengths, segment_slots, heads, qk_heads, dim, vdim)
 #define PICK(RULE)                                                                                                    \
-  if (per <= 4) LAUNCH(4, RULE); else if (per <= 8) LAUNCH(8, RULE); else if (per <= 16) LAUNCH(16, RULE);            \
-  else if (per <= 32) LAUNCH(32, RULE); else if (per <= 64) LAUNCH(64, RULE); else LAUNCH(128, RULE)
+  if (per <= 1) LAUNCH(1, RULE); else if (per <= 2) LAUNCH(2, RULE); else if (per <= 4) LAUNCH(4, RULE);              \
+  else if (per <= 8) LAUNCH(8, RULE); else if (per <= 16) LAUNCH(16, RULE); else LAUNCH(32, RULE)
   if (rule == 0) { PICK(0); } else { PICK(1); }
 #undef PICK
 #undef LAUNCH

@@ -1151,10 +1151,24 @@ def scan_gate(out, z, kind: str, bias=None, per_head=None, head_width: int = 0, 
                     SCAN_GATES[kind], float(number), int(first_columns), n, w, _stream())
 
 
+SCAN_COLUMNS = 4
+
+
+def scan_state_shape(dim: int, vdim: int) -> tuple:
+    """How `linear_scan` keeps a head's matrix S [dim, vdim]: [blocks of four columns, dim, 4]."""
+    return ((vdim + SCAN_COLUMNS - 1) // SCAN_COLUMNS, dim, SCAN_COLUMNS)
+
+
+def scan_state_matrix(state: torch.Tensor, vdim: int) -> torch.Tensor:
+    """[..., blocks, dim, 4] as `linear_scan` keeps it -> [..., dim, vdim]."""
+    s = state.transpose(-3, -2)
+    return s.reshape(*s.shape[:-2], -1)[..., :vdim]
+
+
 def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots, heads: int,
                 qk_heads: int, dim: int, vdim: int, rule: str):
-    """Walks each segment's rows in order from state[slot] ([slots, heads, dim, vdim] float32, updated in
-    place).  rule "decay_add": S <- diag(decay) S + k v^T; "delta": S <- diag(decay) S,
+    """Walks each segment's rows in order from state[slot] (float32 [slots, heads, `scan_state_shape`],
+    updated in place: a head's matrix in blocks of four columns).  rule "decay_add": S <- diag(decay) S + k v^T; "delta": S <- diag(decay) S,
     S <- S + k (beta (v - S^T k))^T; out = S^T q.  q, k: float32 [n, qk_heads * dim] (head h reads
     q/k head h // (heads / qk_heads)); v, out: [n, heads * vdim]; decay: [n, heads * dim]; beta [n, heads]."""
     _gpu(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots)
@@ -1166,8 +1180,8 @@ def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths,
     _check(rule in ("decay_add", "delta"), "linear_scan: rule is 'decay_add' or 'delta'")
     _check(nk == nv == nd == no == n and wq == wk == qk_heads * dim and wv == wo == heads * vdim and wd == heads * dim,
            "linear_scan: shapes")
-    _check(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dim, vdim),
-           "linear_scan: the state must be float32 [slots, heads, dim, vdim]")
+    _check(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, *scan_state_shape(dim, vdim)),
+           "linear_scan: the state must be float32 [slots, heads, *scan_state_shape(dim, vdim)]")
     ldb = 0
     if rule == "delta":
         nb, wb, ldb = _f32rows(beta, "linear_scan beta")

@@ -95,7 +95,7 @@ class GatedDelta(_StateMixer):
         self.w_a_up_tiles, self.w_g_up_tiles = tiles_of(self.dtype, self.w_a_up, self.w_g_up)
 
     def state_specs(self):
-        return [(self.prefix + "state", (self.heads, self.dim, self.vdim), torch.float32),
+        return [(self.prefix + "state", (self.heads, *ops.scan_state_shape(self.dim, self.vdim)), torch.float32),
                 (self.prefix + "conv_state", (self.taps - 1, self.channels), self.dtype)]
 
     def prepare(self, info):
@@ -170,7 +170,7 @@ class GatedLinearAttention(_StateMixer):
         self.w_in_tiles, self.w_o_tiles, self.w_a_up_tiles = tiles_of(self.dtype, self.w_in, self.w_o, self.w_a_up)
 
     def state_specs(self):
-        return [(self.prefix + "state", (self.heads, self.dim, self.vdim), torch.float32)]
+        return [(self.prefix + "state", (self.heads, *ops.scan_state_shape(self.dim, self.vdim)), torch.float32)]
 
     def prepare(self, info):
         self.state = info.storage.states[self.prefix + "state"]

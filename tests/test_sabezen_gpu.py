@@ -153,9 +153,10 @@ def test_linear_scan_in_portions(rule, H, G, D, V):
         a = torch.rand(t, H, D, generator=g) * 0.3 + 0.7
         b = torch.rand(t, H, generator=g)
         data.append((q, k, v, a, b))
-    want = []
+    want, final = [], []
     for q, k, v, a, b in data:
         o = torch.zeros(q.shape[0], H, V, dtype=torch.float64)
+        final.append([])
         for h in range(H):
             S = torch.zeros(D, V, dtype=torch.float64)
             for t in range(q.shape[0]):
@@ -164,8 +165,9 @@ def test_linear_scan_in_portions(rule, H, G, D, V):
                 u = b[t, h].double() * (v[t, h].double() - S.T @ kt) if rule == "delta" else v[t, h].double()
                 S = S + kt[:, None] * u[None, :]
                 o[t, h] = S.T @ qt
+            final[-1].append(S)
         want.append(o.reshape(q.shape[0], -1))
-    state = torch.zeros(5, H, D, V, device="cuda")
+    state = torch.zeros(5, H, *ops.scan_state_shape(D, V), device="cuda")
     state[1].fill_(float("nan"))                    # a slot that nobody uses
     slots = [3, 0]
     fed = [0, 0]
@@ -184,6 +186,8 @@ def test_linear_scan_in_portions(rule, H, G, D, V):
     assert fed == T
     for s in range(2):
         assert su.rel(got[s], want[s]) < 2e-5
+        assert su.rel(ops.scan_state_matrix(state[slots[s]], V).cpu(), torch.stack(final[s])) < 2e-5
+    assert bool(torch.isnan(state[1]).all()) and float(state[2].abs().sum()) == 0.0
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
