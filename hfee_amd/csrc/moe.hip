@@ -7,9 +7,17 @@
 //   up:    act[t][j][f] = silu(W_gate[e][f] . h_t) * (W_up[e][f] . h_t),   e = the j-th expert of t
 //   down:  x[t][c] (+)= sum_j weight_tj (W_down[e_j][c] . act[t][j])
 //
-// A wave a dot product, lanes over the summed dimension, added up in a fixed order; the experts'
-// matrices are stacked [experts][rows][columns].  Every token reads the rows of its own experts:
-// this is the form for steps of few tokens, whose time is the experts' bytes.
+// The experts' matrices are stacked [experts][rows][columns].  Two forms:
+//
+// Token by token (moe_up, moe_down): a wave a dot product, lanes over the summed dimension, added up in a
+// fixed order; every token reads the rows of its own experts.  For steps of few tokens, whose time is
+// the experts' bytes, and for float32.
+//
+// Grouped (moe_group, moe_group_up, moe_group_down, moe_combine; bfloat16): the (token, expert) pairs of a
+// step are put in the order of their experts on the device, cut into tiles of 64 pairs of one expert, and
+// a workgroup multiplies a tile by 256 rows of that expert's matrix on the matrix cores (a wave 64 x 64
+// of v_mfma_f32_16x16x32_bf16, operands straight from memory): an expert's matrices are read once a
+// 64 pairs and not once a pair.  A pair's numbers do not depend on which pairs share its tile.
 #include "common.h"
 
 using namespace hfee;
@@ -22,6 +30,45 @@ __device__ __forceinline__ int expert_of(const int* chosen, const int* table, co
 
 constexpr int kRowsPerWave = 4;
 
+// sum_c a[c] b[c] and sum_c a2[c] b[c] over `count` elements, a lane's share: lanes take turns of one
+// element, or of eight bfloat16 (sixteen bytes) where count is a multiple of eight and the rows are aligned.
+template <typename T>
+__device__ __forceinline__ void two_dots(const T* a, const T* a2, const T* b, int count, int lane, bool wide, float& s, float& s2) {
+  s = s2 = 0.f;
+  if constexpr (sizeof(T) == 2) {
+    if (wide) {
+      typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+      for (int c = lane * 8; c < count; c += 64 * 8) {
+        const u32x4_t va = load_streamed(reinterpret_cast<const u32x4_t*>(a + c));
+        const u32x4_t vb = *reinterpret_cast<const u32x4_t*>(b + c);
+        u32x4_t va2 = va;
+        if (a2 != nullptr) va2 = load_streamed(reinterpret_cast<const u32x4_t*>(a2 + c));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float b0 = __uint_as_float(vb[i] << 16), b1 = __uint_as_float(vb[i] & 0xffff0000u);
+          s = fmaf(__uint_as_float(va[i] << 16), b0, s);
+          s = fmaf(__uint_as_float(va[i] & 0xffff0000u), b1, s);
+          if (a2 != nullptr) {
+            s2 = fmaf(__uint_as_float(va2[i] << 16), b0, s2);
+            s2 = fmaf(__uint_as_float(va2[i] & 0xffff0000u), b1, s2);
+          }
+        }
+      }
+      return;
+    }
+  }
+  for (int c = lane; c < count; c += 64) {
+    const float x = to_float<T>(b[c]);
+    s = fmaf(to_float<T>(a[c]), x, s);
+    if (a2 != nullptr) s2 = fmaf(to_float<T>(a2[c]), x, s2);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ bool rows_aligned(const T* a, const T* b, int count, int64_t row_stride_b) {
+  return sizeof(T) == 2 && count % 8 == 0 && row_stride_b % 8 == 0 && ((uintptr_t)a | (uintptr_t)b) % 16 == 0;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act, const T* __restrict__ h, int64_t ldh,
                                                      const T* __restrict__ w_gate, const T* __restrict__ w_up,
@@ -33,6 +80,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act, const 
   const int e = expert_of(chosen, table, token_ids, t, j, top);
   if (e < 0 || e >= experts) return;                       // (a table that names no such expert: nothing is read)
   const T* hr = h + (int64_t)t * ldh;
+  const bool wide = rows_aligned<T>(w_gate, h, width, ldh) && (uintptr_t)w_up % 16 == 0;
   const int f0 = (blockIdx.y * 4 + wave) * kRowsPerWave;
 #pragma unroll
   for (int r = 0; r < kRowsPerWave; ++r) {
@@ -40,12 +88,8 @@ __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act, const 
     if (f >= F) break;
     const T* g = w_gate + ((int64_t)e * F + f) * width;
     const T* u = w_up + ((int64_t)e * F + f) * width;
-    float sg = 0.f, su = 0.f;
-    for (int c = lane; c < width; c += 64) {
-      const float x = to_float<T>(hr[c]);
-      sg = fmaf(to_float<T>(g[c]), x, sg);
-      su = fmaf(to_float<T>(u[c]), x, su);
-    }
+    float sg, su;
+    two_dots<T>(g, u, hr, width, lane, wide, sg, su);
     sg = wave_sum(sg);
     su = wave_sum(su);
     if (lane == 0) act[(int64_t)pair * F + f] = from_float<T>(sg / (1.0f + expf(-sg)) * su);
@@ -60,6 +104,7 @@ __global__ __launch_bounds__(256) void moe_down_kernel(float* __restrict__ x, in
                                                        int experts, int F, int width, int accumulate) {
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c0 = (blockIdx.y * 4 + wave) * kRowsPerWave;
+  const bool wide = rows_aligned<T>(w_down, act, F, F);
 #pragma unroll
   for (int r = 0; r < kRowsPerWave; ++r) {
     const int c = c0 + r;
@@ -70,8 +115,8 @@ __global__ __launch_bounds__(256) void moe_down_kernel(float* __restrict__ x, in
       if (e < 0 || e >= experts) continue;
       const T* w = w_down + ((int64_t)e * width + c) * F;
       const T* a = act + ((int64_t)t * top + j) * F;
-      float s = 0.f;
-      for (int f = lane; f < F; f += 64) s = fmaf(to_float<T>(w[f]), to_float<T>(a[f]), s);
+      float s, unused;
+      two_dots<T>(w, nullptr, a, F, lane, wide, s, unused);
       total = fmaf(wave_sum(s), pair_weights != nullptr ? pair_weights[(int64_t)t * top + j] : weight, total);
     }
     if (lane == 0) {
@@ -81,7 +126,222 @@ __global__ __launch_bounds__(256) void moe_down_kernel(float* __restrict__ x, in
   }
 }
 
+// ---------------------------------------------------------------------------- grouped
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+union Operand {
+  u32x4 u;
+  bf16x8 v;
+};
+
+constexpr int kTilePairs = 64, kTileRows = 256;
+
+// One workgroup.  order: the pairs (t * top + j) by expert; tiles: (expert, first place in order, pairs)
+// for every tile, tiles[3 * most_tiles] holds their number.  Which of an expert's pairs comes first is
+// left to chance; nothing that is computed depends on it.
+__global__ __launch_bounds__(1024) void moe_group_kernel(int* __restrict__ order, int* __restrict__ tiles, int most_tiles,
+                                                         const int* __restrict__ chosen, const int* __restrict__ table,
+                                                         const int* __restrict__ token_ids, int n, int top, int experts) {
+  extern __shared__ int lds[];
+  int* counts = lds;                  // [experts]
+  int* starts = lds + experts;        // [experts]
+  int* cursor = lds + 2 * experts;    // [experts]
+  int* first_tile = lds + 3 * experts;
+  const int pairs = n * top;
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = cursor[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = expert_of(chosen, table, token_ids, p / top, p % top, top);
+    if (e >= 0 && e < experts) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tile = 0;
+    for (int e = 0; e < experts; ++e) {
+      starts[e] = at;
+      first_tile[e] = tile;
+      at += counts[e];
+      tile += (counts[e] + kTilePairs - 1) / kTilePairs;
+    }
+    tiles[3 * most_tiles] = tile;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+    const int e = expert_of(chosen, table, token_ids, p / top, p % top, top);
+    if (e >= 0 && e < experts) order[starts[e] + atomicAdd(&cursor[e], 1)] = p;
+  }
+  for (int e = threadIdx.x; e < experts; e += blockDim.x)
+    for (int i = 0; i * kTilePairs < counts[e]; ++i) {
+      int* tl = tiles + 3 * (first_tile[e] + i);
+      tl[0] = e;
+      tl[1] = starts[e] + i * kTilePairs;
+      tl[2] = min(kTilePairs, counts[e] - i * kTilePairs);
+    }
+}
+
+// C[64 pairs][64 rows of B] (+)= A B^T for one wave: A rows through a_rows (pointers to the K elements of
+// each of the lane's four pair rows), B rows from b (row stride K; rows at and beyond n_rows read row 0).
+template <int NB>
+__device__ __forceinline__ void tile_products(f32x4 (&acc)[NB][4][4], const bf16_t* const (&a_rows)[4],
+                                              const bf16_t* const (&b)[NB], int64_t K, int row0, int n_rows, int lane) {
+  const int r16 = lane & 15, kg = (lane >> 4) * 8;
+  const bf16_t* b_rows[NB][4];
+#pragma unroll
+  for (int m = 0; m < NB; ++m)
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int row = row0 + nt * 16 + r16;
+      b_rows[m][nt] = b[m] + (int64_t)(row < n_rows ? row : 0) * K + kg;
+    }
+  for (int64_t k0 = 0; k0 < K; k0 += 32) {
+    Operand a[4], w[NB][4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) a[mt].u = *reinterpret_cast<const u32x4*>(a_rows[mt] + k0 + kg);
+#pragma unroll
+    for (int m = 0; m < NB; ++m)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) w[m][nt].u = *reinterpret_cast<const u32x4*>(b_rows[m][nt] + k0);
+#pragma unroll
+    for (int m = 0; m < NB; ++m)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+          acc[m][nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[m][nt].v, a[mt].v, acc[m][nt][mt], 0, 0, 0);
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_group_up_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ h, int64_t ldh,
+                                                           const bf16_t* __restrict__ w_gate, const bf16_t* __restrict__ w_up,
+                                                           const int* __restrict__ order, const int* __restrict__ tiles,
+                                                           int most_tiles, int top, int F, int width) {
+  if ((int)blockIdx.x >= tiles[3 * most_tiles]) return;
+  const int* tl = tiles + 3 * blockIdx.x;
+  const int e = tl[0], first = tl[1], count = tl[2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15;
+  const int row0 = blockIdx.y * kTileRows + wave * 64;
+  if (row0 >= F) return;
+  int pair[4];
+  const bf16_t* a_rows[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int r = mt * 16 + r16;
+    pair[mt] = order[first + (r < count ? r : 0)];
+    a_rows[mt] = h + (int64_t)(pair[mt] / top) * ldh;
+  }
+  const bf16_t* const b[2] = {w_gate + (int64_t)e * F * width, w_up + (int64_t)e * F * width};
+  f32x4 acc[2][4][4] = {};
+  tile_products<2>(acc, a_rows, b, width, row0, F, lane);
+  // register i of lane l: row of the matrix 16 nt + 4 (l / 16) + i, pair row 16 mt + l % 16
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    if (mt * 16 + r16 >= count) continue;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int f = row0 + nt * 16 + (lane >> 4) * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float g = acc[0][nt][mt][i];
+        if (f + i < F) act[(int64_t)pair[mt] * F + f + i] = float_to_bf16(g / (1.0f + expf(-g)) * acc[1][nt][mt][i]);
+      }
+    }
+  }
+}
+
+// out: x (float32 [n, width]) when a token has one expert (then out[t] += weight * product), else
+// y (float32 [pairs, width]) = product.
+__global__ __launch_bounds__(256) void moe_group_down_kernel(float* __restrict__ out, int64_t ldo, const bf16_t* __restrict__ act,
+                                                             const bf16_t* __restrict__ w_down, const int* __restrict__ order,
+                                                             const int* __restrict__ tiles, int most_tiles, int F, int width,
+                                                             int add, const float* __restrict__ pair_weights, float weight) {
+  if ((int)blockIdx.x >= tiles[3 * most_tiles]) return;
+  const int* tl = tiles + 3 * blockIdx.x;
+  const int e = tl[0], first = tl[1], count = tl[2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15;
+  const int row0 = blockIdx.y * kTileRows + wave * 64;
+  if (row0 >= width) return;
+  int pair[4];
+  const bf16_t* a_rows[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int r = mt * 16 + r16;
+    pair[mt] = order[first + (r < count ? r : 0)];
+    a_rows[mt] = act + (int64_t)pair[mt] * F;
+  }
+  const bf16_t* const b[1] = {w_down + (int64_t)e * width * F};
+  f32x4 acc[1][4][4] = {};
+  tile_products<1>(acc, a_rows, b, F, row0, width, lane);
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    if (mt * 16 + r16 >= count) continue;
+    const float scale = add ? (pair_weights != nullptr ? pair_weights[pair[mt]] : weight) : 1.0f;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int c = row0 + nt * 16 + (lane >> 4) * 4;
+      float* o = out + (int64_t)pair[mt] * ldo + c;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (c + i < width) o[i] = add ? fmaf(acc[0][nt][mt][i], scale, o[i]) : acc[0][nt][mt][i];
+    }
+  }
+}
+
+// x[t] += sum_j weight_tj y[t * top + j], j ascending.
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, int64_t ldx, const float* __restrict__ y,
+                                                          const float* __restrict__ pair_weights, float weight, int top,
+                                                          int width) {
+  const int64_t t = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
+    float total = 0.f;
+    for (int j = 0; j < top; ++j)
+      total = fmaf(y[(t * top + j) * width + c], pair_weights != nullptr ? pair_weights[t * top + j] : weight, total);
+    x[t * ldx + c] += total;
+  }
+}
+
 }  // namespace
+
+// The whole feed-forward in its grouped form, bfloat16: x (float32 [n, width]) += the experts' weighted
+// outputs.  order: int32 [n * top]; tiles: int32 [3 * hfee_moe_group_tiles(n, top, experts) + 1]; act:
+// bfloat16 [n * top, ff]; y: float32 [n * top, width], needed where top > 1.
+HFEE_API int hfee_moe_group_tiles(int n, int top, int experts) {
+  return (int)(((int64_t)n * top + kTilePairs - 1) / kTilePairs) + experts;
+}
+
+HFEE_API int hfee_moe_grouped(float* x, int64_t ldx, const void* h, int64_t ldh, const void* w_gate, const void* w_up,
+                              const void* w_down, const int* chosen, const int* table, const int* token_ids,
+                              const float* pair_weights, float weight, int top, int experts, int ff, int width, int n,
+                              int* order, int* tiles, void* act, float* y, hipStream_t stream) {
+  HFEE_REQUIRE(n >= 0 && top >= 1 && experts >= 1 && experts <= 8192 && ff >= 1 && width >= 1, "moe_grouped: bad sizes");
+  HFEE_REQUIRE(chosen != nullptr || (table != nullptr && token_ids != nullptr), "moe_grouped: the experts of a token, or a table and the ids");
+  HFEE_REQUIRE(width % 32 == 0 && ff % 32 == 0 && ldh % 8 == 0 && ldx >= width && ldh >= width,
+               "moe_grouped: the width and the experts' size must be multiples of 32");
+  HFEE_REQUIRE(((uintptr_t)h | (uintptr_t)w_gate | (uintptr_t)w_up | (uintptr_t)w_down | (uintptr_t)act) % 16 == 0,
+               "moe_grouped: operands must be 16-byte aligned");
+  HFEE_REQUIRE(order != nullptr && tiles != nullptr && act != nullptr && (top == 1 || y != nullptr), "moe_grouped: scratch missing");
+  HFEE_REQUIRE((int64_t)n * top < (1 << 30), "moe_grouped: too many pairs");
+  if (n == 0) return 0;
+  const int most = hfee_moe_group_tiles(n, top, experts);
+  moe_group_kernel<<<1, 1024, 4 * experts * sizeof(int), stream>>>(order, tiles, most, chosen, table, token_ids, n, top, experts);
+  HFEE_CHECK_LAUNCH("moe_group");
+  moe_group_up_kernel<<<dim3(most, (ff + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
+      (bf16_t*)act, (const bf16_t*)h, ldh, (const bf16_t*)w_gate, (const bf16_t*)w_up, order, tiles, most, top, ff, width);
+  HFEE_CHECK_LAUNCH("moe_group_up");
+  moe_group_down_kernel<<<dim3(most, (width + kTileRows - 1) / kTileRows), 256, 0, stream>>>(
+      top == 1 ? x : y, top == 1 ? ldx : (int64_t)width, (const bf16_t*)act, (const bf16_t*)w_down, order, tiles, most, ff, width,
+      top == 1 ? 1 : 0, pair_weights, weight);
+  HFEE_CHECK_LAUNCH("moe_group_down");
+  if (top > 1) {
+    int parts = (width + 255) / 256;
+    if (parts > 64) parts = 64;
+    moe_combine_kernel<<<dim3(n, parts), 256, 0, stream>>>(x, ldx, y, pair_weights, weight, top, width);
+    HFEE_CHECK_LAUNCH("moe_combine");
+  }
+  return 0;
+}
 
 HFEE_API int hfee_moe_up(void* act, const void* h, int64_t ldh, const void* w_gate, const void* w_up, int dtype,
                          const int* chosen, const int* table, const int* token_ids, int top, int experts, int ff,

@@ -134,11 +134,19 @@ __device__ __forceinline__ void scan_load(ScanInputs<DPT>& in, const float* __re
   in.b = RULE == 1 ? beta[(int64_t)t * ldb + h] : 1.f;
 }
 
-__device__ __forceinline__ float column_sum(float x) {      // over the sixteen lanes of a column
-  x += __shfl_xor(x, 1, kWave);
-  x += __shfl_xor(x, 2, kWave);
-  x += __shfl_xor(x, 4, kWave);
-  x += __shfl_xor(x, 8, kWave);
+// Over the sixteen lanes of a column, which are one row of the data-parallel primitives: neighbours in a
+// quad, the quads of a half, the halves.  Every step adds two numbers that both lanes of a pair hold the
+// other way round, so all sixteen lanes end with the same bits.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ float column_sum(float x) {
+  x += dpp_move<0xB1>(x);      // quad_perm [1, 0, 3, 2]
+  x += dpp_move<0x4E>(x);      // quad_perm [2, 3, 0, 1]
+  x += dpp_move<0x141>(x);     // row_half_mirror: lane i of eight reads lane 7 - i
+  x += dpp_move<0x140>(x);     // row_mirror: lane i of sixteen reads lane 15 - i
   return x;
 }
 

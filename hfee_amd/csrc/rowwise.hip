@@ -174,6 +174,9 @@ __global__ __launch_bounds__(256) void rmsnorm_cols_kernel(T* __restrict__ out, 
 
 // x float32 [rows, d]; row r of out is made from row rows[r] (or r) of x.  The mean first, then the
 // mean of the squared deviations from it, both as sums over the workgroup in a fixed order.
+// Rows of up to 16 values a thread stay in registers between the three passes; wider rows are read again.
+constexpr int kLayerNormKeep = 16;
+
 template <typename TO, typename TW>
 __global__ __launch_bounds__(256) void layernorm_kernel(TO* __restrict__ out, const float* __restrict__ x,
                                                         const TW* __restrict__ w, const int* __restrict__ rows,
@@ -181,6 +184,33 @@ __global__ __launch_bounds__(256) void layernorm_kernel(TO* __restrict__ out, co
   __shared__ float scratch[16];
   const int64_t r = blockIdx.x;
   const float* xr = x + (int64_t)(rows ? rows[r] : r) * d;
+  TO* o = out + r * d;
+  if (d <= kLayerNormKeep * 256) {
+    float v[kLayerNormKeep], wv[kLayerNormKeep];
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < kLayerNormKeep; ++i) {
+      const int j = threadIdx.x + i * 256;
+      v[i] = j < d ? xr[j] : 0.f;
+      wv[i] = j < d ? to_float<TW>(w[j]) : 0.f;
+      sum += v[i];
+    }
+    const float mean = block_sum(sum, scratch) / (float)d;
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < kLayerNormKeep; ++i) {
+      const int j = threadIdx.x + i * 256;
+      v[i] = j < d ? v[i] - mean : 0.f;
+      ss = fmaf(v[i], v[i], ss);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)d + eps);
+#pragma unroll
+    for (int i = 0; i < kLayerNormKeep; ++i) {
+      const int j = threadIdx.x + i * 256;
+      if (j < d) o[j] = from_float<TO>(v[i] * inv * wv[i]);
+    }
+    return;
+  }
   float sum = 0.f;
   for (int j = threadIdx.x; j < d; j += blockDim.x) sum += xr[j];
   const float mean = block_sum(sum, scratch) / (float)d;
@@ -190,7 +220,6 @@ __global__ __launch_bounds__(256) void layernorm_kernel(TO* __restrict__ out, co
     ss = fmaf(v, v, ss);
   }
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)d + eps);
-  TO* o = out + r * d;
   for (int j = threadIdx.x; j < d; j += blockDim.x) o[j] = from_float<TO>((xr[j] - mean) * inv * to_float<TW>(w[j]));
 }
 

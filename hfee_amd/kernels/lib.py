@@ -61,6 +61,7 @@ _CORE_SIGNATURES = {
     "hfee_scan_gate": [P, L, P, L, I, P, P, I, I, F, I, I, I, P],
     "hfee_linear_scan": [P, L, P, P, L, P, L, P, L, P, L, P, L, P, P, P, I, I, I, I, I, I, P],
     "hfee_head_norm_gate": [P, L, P, L, P, L, I, P, I, I, F, I, I, P],
+    "hfee_moe_grouped": [P, L, P, L, P, P, P, P, P, P, P, F, I, I, I, I, I, P, P, P, P, P],
     "hfee_moe_up": [P, P, L, P, P, I, P, P, P, I, I, I, I, I, P],
     "hfee_moe_down": [P, L, P, P, I, P, P, P, P, F, I, I, I, I, I, I, P],
     "hfee_rmsnorm_cols": [P, L, P, L, I, P, I, F, F, I, I, P],

@@ -1249,3 +1249,43 @@ def moe_down(x, act, w_down, top: int, weight: float = 1.0, pair_weights=None, c
     _experts_of(chosen, table, token_ids, n, top, "moe_down")
     lib.core().call("hfee_moe_down", _ptr(x), ldx, _ptr(act), _ptr(w_down), _dt(act), _ptr(chosen), _ptr(table),
                     _ptr(token_ids), _ptr(pair_weights), float(weight), top, E, F, width, 1 if accumulate else 0, n, _stream())
+
+
+MOE_TILE_PAIRS = 64
+
+
+def moe_group_tiles(n: int, top: int, experts: int) -> int:
+    """The most tiles of 64 (token, expert) pairs of one expert that a step of n tokens can make."""
+    return (n * top + MOE_TILE_PAIRS - 1) // MOE_TILE_PAIRS + experts
+
+
+def moe_grouped_fits(dtype, width: int, ff: int) -> bool:
+    return dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
+
+
+def moe_grouped(x, h, w_gate, w_up, w_down, top: int, order, tiles, act, y=None, weight: float = 1.0, pair_weights=None,
+                chosen=None, table=None, token_ids=None):
+    """x[t] += sum_j weight_tj * w_down[e_j] @ (silu(w_gate[e_j] @ h[t]) * (w_up[e_j] @ h[t])), bfloat16, with the
+    step's (token, expert) pairs grouped by expert on the device and multiplied in tiles on the matrix cores.
+    order: int32 [n * top]; tiles: int32 [3 * moe_group_tiles(n, top, experts) + 1]; act: bfloat16
+    [n * top, ff]; y: float32 [n * top, width] (where top > 1): scratch."""
+    _gpu(x, h, w_gate, w_up, w_down, order, tiles, act, y, pair_weights, chosen, table, token_ids)
+    n, width, ldh = _rows2d(h, "moe_grouped h")
+    nx, wx, ldx = _f32rows(x, "moe_grouped x")
+    E, F, W = w_gate.shape
+    _check(nx == n and wx == width == W and w_up.shape == w_gate.shape and tuple(w_down.shape) == (E, width, F)
+           and w_gate.is_contiguous() and w_up.is_contiguous() and w_down.is_contiguous(), "moe_grouped: shapes")
+    _check(h.dtype == w_gate.dtype == w_up.dtype == w_down.dtype == act.dtype == torch.bfloat16, "moe_grouped: bfloat16 operands")
+    _check(act.is_contiguous() and act.numel() >= n * top * F, "moe_grouped: act [n * top, ff]")
+    _check(order.dtype == tiles.dtype == torch.int32 and order.is_contiguous() and tiles.is_contiguous()
+           and order.numel() >= n * top and tiles.numel() >= 3 * moe_group_tiles(n, top, E) + 1, "moe_grouped: order and tiles")
+    if top > 1:
+        _check(y is not None and y.dtype == torch.float32 and y.is_contiguous() and y.numel() >= n * top * width,
+               "moe_grouped: y float32 [n * top, width]")
+    if pair_weights is not None:
+        _check(pair_weights.dtype == torch.float32 and pair_weights.is_contiguous() and tuple(pair_weights.shape) == (n, top),
+               "moe_grouped: pair_weights float32 [n, top]")
+    _experts_of(chosen, table, token_ids, n, top, "moe_grouped")
+    lib.core().call("hfee_moe_grouped", _ptr(x), ldx, _ptr(h), ldh, _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(chosen),
+                    _ptr(table), _ptr(token_ids), _ptr(pair_weights), float(weight), top, E, F, width, n, _ptr(order),
+                    _ptr(tiles), _ptr(act), _ptr(y), _stream())

@@ -4,7 +4,10 @@
 entries of a row differ); each counts 1 / top.  Expert: down(act(gate(h)) * up(h)), act the SiLU, no
 biases; the output is the weighted sum of the chosen experts' outputs, added to the residual stream in
 float32.  The experts' matrices are stacked [experts, rows, columns] when they are bound; the lookup
-runs on the device from the step's token ids, so a step may be replayed from a recorded graph.
+runs on the device from the step's token ids, so a step may be replayed from a recorded graph.  A step
+with more (token, expert) pairs than experts groups the pairs by expert on the device and multiplies them
+in tiles on the matrix cores (bfloat16, sizes that are multiples of 32); a step of few tokens, and
+float32, reads each token's experts row by row.
 """
 from __future__ import annotations
 
@@ -60,6 +63,18 @@ class TableMoE(FeedForward):
 
     def forward_add(self, ctx, x, h):
         hn = h.tensor() if isinstance(h, LazyNorm) else h
+        n, top = ctx.n, self.top
+        # more pairs than experts: grouped by expert, an expert's matrices are read once for all its tokens
+        if n * top > self.experts and ops.moe_grouped_fits(self.dtype, self.hidden, self.intermediate) \
+                and hn.data_ptr() % 16 == 0 and hn.stride(0) % 8 == 0:
+            ws = ctx.workspace
+            order = ws.flat("table_moe.order", ws.capacity * top, torch.int32)
+            tiles = ws.flat("table_moe.tiles", 3 * ops.moe_group_tiles(ws.capacity, top, self.experts) + 1, torch.int32)
+            act = ctx.rows("table_moe.act", top * self.intermediate)
+            y = ctx.rows("table_moe.rows", top * self.hidden, torch.float32) if top > 1 else None
+            ops.moe_grouped(x, hn, self.w_gate, self.w_up, self.w_down, top, order, tiles, act, y, weight=1.0 / top,
+                            table=self.table, token_ids=ctx.token_ids)
+            return
         act = ctx.rows("table_moe.act", self.top * self.intermediate).view(ctx.n * self.top, self.intermediate)
         ops.moe_up(act, hn, self.w_gate, self.w_up, self.top, table=self.table, token_ids=ctx.token_ids)
         ops.moe_down(x, act, self.w_down, self.top, weight=1.0 / self.top, table=self.table, token_ids=ctx.token_ids)

@@ -63,12 +63,13 @@ S_C = config(60, 48, 1e-6, 2.0, [
     moe(gla(3, 8, 24, 16.0, 4), 32, 6, 3),
     bare(delta(2, 2, 16, 16, 5, 8, 8)),
 ])
-# larger, for prompts of hundreds of tokens over many chunks; chunks longer than a tile of keys
+# larger, for prompts of hundreds of tokens over many chunks; chunks longer than a tile of keys; experts of
+# sizes that the grouped kernels take
 S_D = config(500, 128, 1e-6, 8.0, [
     dense(attention(8, 2, 32, 16, 80, 0.15), 160),
-    moe(delta(2, 2, 32, 64, 3, 16, 24), 48, 8, 1),
+    moe(delta(2, 2, 32, 64, 3, 16, 24), 64, 8, 1),
     dense(gla(4, 32, 32, 12.0, 16), 96),
-    moe(attention(8, 2, 32, 16, 80, 0.15), 48, 8, 2),
+    moe(attention(8, 2, 32, 16, 80, 0.15), 96, 8, 2),
 ])
 CONFIGS = {"A": S_A, "B": S_B, "C": S_C, "D": S_D}
 

@@ -236,6 +236,42 @@ def test_experts_by_table(dtype):
     assert su.rel(x.double().cpu() - 1.0, want) < (1e-5 if dtype == "float32" else 2e-2)
 
 
+@pytest.mark.parametrize("n,top,E,F,width", [(300, 2, 5, 96, 64), (70, 1, 3, 32, 96), (9, 3, 4, 64, 32), (129, 4, 40, 320, 128)])
+def test_experts_grouped_on_the_matrix_cores(n, top, E, F, width):
+    """Pairs grouped by expert against the token-by-token kernels and the plain sum: experts with no
+    token, with one, with more than a tile of 64; every token's own result whatever shares its tile."""
+    from hfee_amd.kernels import ops
+    g = torch.Generator().manual_seed(n)
+    vocab = 50
+    h = torch.randn(n, width, generator=g).bfloat16()
+    wg, wu = (torch.randn(E, F, width, generator=g) * 0.2).bfloat16(), (torch.randn(E, F, width, generator=g) * 0.2).bfloat16()
+    wd = (torch.randn(E, width, F, generator=g) * 0.2).bfloat16()
+    table = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(vocab)]).to(torch.int32)
+    if E > 4:
+        table[table == 1] = 0 if top == 1 else table[table == 1]        # (an expert that nobody uses, where rows stay distinct)
+    ids = torch.randint(0, vocab, (n,), generator=g)
+    x0 = torch.randn(n, width, generator=g)
+    one = x0.clone().cuda()
+    act = torch.zeros(n * top, F, dtype=torch.bfloat16, device="cuda")
+    ops.moe_up(act, h.cuda(), wg.cuda(), wu.cuda(), top, table=table.cuda(), token_ids=i32(ids))
+    ops.moe_down(one, act, wd.cuda(), top, weight=1.0 / top, table=table.cuda(), token_ids=i32(ids))
+    grouped = x0.clone().cuda()
+    order = torch.zeros(n * top, dtype=torch.int32, device="cuda")
+    tiles = torch.zeros(3 * ops.moe_group_tiles(n, top, E) + 1, dtype=torch.int32, device="cuda")
+    act2 = torch.zeros(n * top, F, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros(n * top, width, device="cuda") if top > 1 else None
+    ops.moe_grouped(grouped, h.cuda(), wg.cuda(), wu.cuda(), wd.cuda(), top, order, tiles, act2, y, weight=1.0 / top,
+                    table=table.cuda(), token_ids=i32(ids))
+    assert sorted(order.cpu().tolist()) == list(range(n * top))
+    assert su.rel((grouped - x0.cuda()).cpu(), (one - x0.cuda()).cpu()) < 1e-2
+    # the same tokens in another company: a token's numbers stay what they were, bit for bit
+    keep = torch.arange(0, n, 3)
+    again = x0[keep].clone().cuda()
+    ops.moe_grouped(again, h[keep].cuda().contiguous(), wg.cuda(), wu.cuda(), wd.cuda(), top, order, tiles, act2, y,
+                    weight=1.0 / top, table=table.cuda(), token_ids=i32(ids[keep]))
+    assert torch.equal(again.cpu(), grouped.cpu()[keep])
+
+
 # ------------------------------------------------------------------ the whole model
 
 @pytest.fixture(scope="module")
