@@ -10,26 +10,22 @@
 //             denominator may hold one more term exp(sink_h) without a value (a learned number a
 //             head, or zero); out_h = sum_j p_h(j) v_kv(h)(j).
 //
-// The cache layer here is [pages][kv_heads][page_size][2 D]: a slot's scored key, then its value.
+// The cache layer here is that of attention with key and value sizes of their own (`KvLayout`), both
+// sizes D: [pages][kv_heads][page_size * 2 D], the scored keys of a (page, head) as [slot][D], then the
+// values transposed as [D][slot].
 //
 // One workgroup a token takes all heads, since every head's weights need every head's scores.
 // Keys are taken in tiles of 64 counted from first(p), so which thread adds which term in which
 // order depends on positions only: a token's result does not change with the way its sequence
 // was cut into steps, with the batch around it or with page numbers.  Everything is summed in
 // float32; prompt portions and single tokens run the same kernel.
-#include "common.h"
+#include "attention_kv.h"
 
 using namespace hfee;
 
 namespace {
 
-struct MixLayout {
-  int64_t page_stride;   // kv_heads * page_size * 2 * dim
-  int kv_heads, dim, page_size, page_shift;
-  __device__ __forceinline__ int64_t slot_offset(int page, int kvh, int slot) const {
-    return (int64_t)page * page_stride + ((int64_t)kvh * page_size + slot) * 2 * dim;
-  }
-};
+typedef KvLayout MixLayout;      // dk = dv = the head's size
 
 constexpr int kPerLane = 8;     // heads of up to 512 dims: a lane holds dims lane, lane + 64, ...
 
@@ -42,7 +38,7 @@ __global__ __launch_bounds__(256) void mix_prepare_kernel(
     T* __restrict__ cache, MixLayout lay) {
   const int t = blockIdx.x, lane = threadIdx.x & 63;
   const int wave = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6), waves = gridDim.y * (blockDim.x >> 6);
-  const int pos = positions[t], D = lay.dim;
+  const int pos = positions[t], D = lay.dk;
   const float* c = cos_t + (int64_t)pos * half;
   const float* s = sin_t + (int64_t)pos * half;
   const int rows = num_heads + (k != nullptr ? lay.kv_heads : 0);
@@ -76,13 +72,13 @@ __global__ __launch_bounds__(256) void mix_prepare_kernel(
       }
     } else {
       const int page = block_tables[(int64_t)token_segment[t] * bt_stride + (pos >> lay.page_shift)];
-      T* dst = cache + lay.slot_offset(page, row - num_heads, pos & (lay.page_size - 1));
+      const int kvh = row - num_heads, slot = pos & (lay.page_size - 1);
 #pragma unroll
       for (int r = 0; r < kPerLane; ++r) {
         const int d = lane + 64 * r;
         if (d < D) {
-          dst[d] = finite_for_cache<T>(from_float<T>(turned[r] * inv));
-          dst[D + d] = finite_for_cache<T>(from_float<T>(own[r]));
+          cache[lay.key_offset(page, kvh, slot, d)] = finite_for_cache<T>(from_float<T>(turned[r] * inv));
+          cache[lay.value_offset(page, kvh, slot, d)] = finite_for_cache<T>(from_float<T>(own[r]));
         }
       }
     }
@@ -100,7 +96,7 @@ __global__ __launch_bounds__(1024) void mix_attend_kernel(
     int bt_stride, int num_heads, float scale, const float* __restrict__ mix, int chunk, int sink_mode,
     const float* __restrict__ sinks) {
   extern __shared__ float lds[];
-  const int H = num_heads, D = lay.dim, tid = threadIdx.x, threads = blockDim.x;
+  const int H = num_heads, D = lay.dk, tid = threadIdx.x, threads = blockDim.x;
   float* qs = lds;                         // [H][D]
   float* ms = qs + H * D;                  // [H][H] (unused without a mix)
   float* raw = ms + H * H;                 // [H][64]
@@ -134,7 +130,7 @@ __global__ __launch_bounds__(1024) void mix_attend_kernel(
       float sc = 0.f;
       if (jj < count) {
         const int j = j0 + jj;
-        const T* kr = cache + lay.slot_offset(bt[j >> lay.page_shift], g / per_kv, j & (lay.page_size - 1));
+        const T* kr = cache + lay.key_offset(bt[j >> lay.page_shift], g / per_kv, j & (lay.page_size - 1), 0);
         const float* qg = qs + g * D;
         for (int d = 0; d < D; ++d) sc = fmaf(qg[d], to_float<T>(kr[d]), sc);
         sc *= scale;
@@ -177,8 +173,7 @@ __global__ __launch_bounds__(1024) void mix_attend_kernel(
         const float* w = es + h * kKeyTile;
         for (int jj = 0; jj < count; ++jj) {
           const int j = j0 + jj;
-          const T* vr = cache + lay.slot_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1)) + D;
-          o = fmaf(w[jj], to_float<T>(vr[d]), o);
+          o = fmaf(w[jj], to_float<T>(cache[lay.value_offset(bt[j >> lay.page_shift], kvh, j & (lay.page_size - 1), d)]), o);
         }
         acc[r] = o;
       }
@@ -193,16 +188,7 @@ __global__ __launch_bounds__(1024) void mix_attend_kernel(
 }
 
 int make_mix_layout(MixLayout* lay, int kv_heads, int dim, int page_size) {
-  if (page_size < 16 || (page_size & (page_size - 1)) != 0) return fail("page_size must be a power of two >= 16, got %d", page_size);
-  if (kv_heads < 1 || dim < 1) return fail("bad cache shape: kv_heads %d dim %d", kv_heads, dim);
-  lay->kv_heads = kv_heads;
-  lay->dim = dim;
-  lay->page_size = page_size;
-  lay->page_stride = (int64_t)kv_heads * page_size * 2 * dim;
-  int s = 0;
-  while ((1 << s) < page_size) ++s;
-  lay->page_shift = s;
-  return 0;
+  return make_kv_layout(lay, kv_heads, dim, dim, page_size);
 }
 
 }  // namespace

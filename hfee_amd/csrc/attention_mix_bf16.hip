@@ -1,0 +1,200 @@
+// Attention whose heads' scores are mixed before the softmax, on the matrix cores; bfloat16, compiled
+// for one number of heads H (HFEE_MIX_HEADS, a multiple of 4) and one head size D (HFEE_MIX_DIM, a
+// multiple of 32).  What is computed is what attention_mix.hip computes (keys of the query's chunk up to
+// the query, scores of all heads mixed by a matrix, an optional sink, the keys as projected for values).
+//
+// A workgroup of four waves takes an item: up to 16 consecutive rows of one sequence that lie in one
+// chunk, and all heads, a wave H/4 of them.  Keys come in tiles of 16 that start at multiples of 16 of
+// the sequence's positions (a tile lies in one page; keys before the chunk are masked), so what is added
+// in which order depends on positions only.  A tile's steps:
+//   1. raw scores: v_mfma_f32_16x16x32_bf16, the tile's keys as the first operand straight from the
+//      page, the rows' queries (held in registers for all tiles) as the second; lane l then holds, for
+//      row l % 16, the keys 4 (l / 16) .. + 3: sixteen bytes of raw[head][row][key] in LDS.
+//   2. mixing on the vector units in float32: the wave's heads h, s_h = sum_g T[h][g] raw_g for the lane's
+//      row and four keys; T comes transposed ([g][h]) through scalar loads, the same for all lanes.
+//   3. the softmax's running maximum and sum for each (head, row), over the lane's four keys and the
+//      four lanes of a row; the weights rounded to bfloat16 are, as they lie, the second operand of
+//   4. v_mfma_f32_16x16x16_bf16 with four keys of a value column (8 bytes of the page) as the first:
+//      out[head][16 dims][row] a register block.
+// A single token is an item of one row.
+#include "attention_kv.h"
+
+using namespace hfee;
+
+#ifndef HFEE_MIX_HEADS
+#error "compile with -DHFEE_MIX_HEADS=<heads> -DHFEE_MIX_DIM=<head size>"
+#endif
+
+namespace {
+
+constexpr int H = HFEE_MIX_HEADS, D = HFEE_MIX_DIM;
+constexpr int WAVES = 4, HW = H / WAVES, KS = D / 32, DB = D / 16, ROWS = 16, KEYS = 16;
+static_assert(H % WAVES == 0 && D % 32 == 0, "heads in fours, head sizes in multiples of 32");
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+union Operand8 {
+  u32x4 u;
+  bf16x8 v;
+};
+union Operand4 {
+  u32x2 u;
+  s16x4 v;
+};
+
+__global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
+    bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq, const bf16_t* __restrict__ cache,
+    KvLayout lay, const int* __restrict__ items, const int* __restrict__ block_tables, int bt_stride, float scale,
+    const float* __restrict__ mix_t, int chunk, int sink_mode, const float* __restrict__ sinks) {
+  __shared__ float raw[H][ROWS][KEYS];
+  const int4 item = reinterpret_cast<const int4*>(items)[blockIdx.x];
+  const int row0 = item.x, rows = item.y, p0 = item.z;
+  const int* bt = block_tables + (int64_t)item.w * bt_stride;
+  const int lane = threadIdx.x & 63, r16 = lane & 15, kq = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int first = chunk > 0 ? p0 / chunk * chunk : 0, last = p0 + rows - 1;
+  const int per_kv = H / lay.kv_heads;
+  const int my_row = r16 < rows ? r16 : rows - 1;
+
+  Operand8 qop[HW][KS];
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qop[hh][ks].u = *reinterpret_cast<const u32x4*>(q + (int64_t)(row0 + my_row) * ldq + (wave * HW + hh) * D + ks * 32 + kq * 8);
+
+  f32x4 o[HW][DB];
+  float m[HW], l[HW];
+#pragma unroll
+  for (int hh = 0; hh < HW; ++hh) {
+    m[hh] = sink_mode == 0 ? -INFINITY : sink_mode == 1 ? 0.f : sinks[wave * HW + hh];
+    l[hh] = sink_mode == 0 ? 0.f : 1.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o[hh][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int j0 = first & ~(KEYS - 1); j0 <= last; j0 += KEYS) {
+    const int page = bt[j0 >> lay.page_shift], slot0 = j0 & (lay.page_size - 1);
+    // 1. raw scores of the wave's heads
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      const int g = wave * HW + hh;
+      const bf16_t* kr = cache + lay.key_offset(page, g / per_kv, slot0 + r16, kq * 8);
+      f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Operand8 kop;
+        kop.u = *reinterpret_cast<const u32x4*>(kr + ks * 32);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qop[hh][ks].v, s, 0, 0, 0);
+      }
+      *reinterpret_cast<f32x4*>(&raw[g][r16][kq * 4]) = s * scale;
+    }
+    __syncthreads();
+    // 2. the scores that enter the softmax
+    f32x4 sc[HW];
+    if (mix_t != nullptr) {
+#pragma unroll
+      for (int hh = 0; hh < HW; ++hh) sc[hh] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const float* tw = mix_t + wave * HW;
+#pragma unroll 4
+      for (int g = 0; g < H; ++g) {
+        const f32x4 r = *reinterpret_cast<const f32x4*>(&raw[g][r16][kq * 4]);
+#pragma unroll
+        for (int hh = 0; hh < HW; ++hh) {
+          const float w = tw[g * H + hh];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) sc[hh][i] = fmaf(w, r[i], sc[hh][i]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int hh = 0; hh < HW; ++hh) sc[hh] = *reinterpret_cast<const f32x4*>(&raw[wave * HW + hh][r16][kq * 4]);
+    }
+    __syncthreads();
+    // 3. and 4. head by head
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      const int kvh = (wave * HW + hh) / per_kv;
+      float tmax = -INFINITY;
+      bool seen[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = j0 + kq * 4 + i;
+        seen[i] = j >= first && j <= p0 + r16 && r16 < rows;
+        if (seen[i]) tmax = fmaxf(tmax, sc[hh][i]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+      const float m_new = fmaxf(m[hh], tmax);
+      float p[4], psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = seen[i] ? expf(sc[hh][i] - m_new) : 0.f;
+        psum += p[i];
+      }
+      psum += __shfl_xor(psum, 16, kWave);
+      psum += __shfl_xor(psum, 32, kWave);
+      const float shrink = m[hh] == -INFINITY ? 0.f : expf(m[hh] - m_new);      // (m_new is finite wherever m is)
+      l[hh] = fmaf(l[hh], shrink, psum);
+      m[hh] = m_new;
+      Operand4 pop;
+      pop.u = u32x2{(uint32_t)float_to_bf16(p[0]) | ((uint32_t)float_to_bf16(p[1]) << 16),
+                    (uint32_t)float_to_bf16(p[2]) | ((uint32_t)float_to_bf16(p[3]) << 16)};
+      const bf16_t* vr = cache + lay.value_offset(page, kvh, slot0 + kq * 4, r16);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        Operand4 vop;
+        vop.u = *reinterpret_cast<const u32x2*>(vr + (int64_t)db * 16 * lay.page_size);
+        o[hh][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop.v, pop.v, o[hh][db] * shrink, 0, 0, 0);
+      }
+    }
+  }
+  // register i of lane l: dim 16 db + 4 (l / 16) + i of row l % 16
+  if (r16 < rows) {
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      const float inv = 1.0f / l[hh];
+      bf16_t* dst = out + (int64_t)(row0 + r16) * ld_out + (wave * HW + hh) * D + kq * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const f32x4 v = o[hh][db] * inv;
+        *reinterpret_cast<u32x2*>(dst + db * 16) = u32x2{(uint32_t)float_to_bf16(v[0]) | ((uint32_t)float_to_bf16(v[1]) << 16),
+                                                        (uint32_t)float_to_bf16(v[2]) | ((uint32_t)float_to_bf16(v[3]) << 16)};
+      }
+    }
+  }
+}
+
+}  // namespace
+
+HFEE_DEFINE_LAST_ERROR
+
+HFEE_API int hfee_attention_mix_bf16_heads() { return H; }
+HFEE_API int hfee_attention_mix_bf16_dim() { return D; }
+
+// items: int32 [count][4] on the device: first row, rows (1..16), first position, block-table row; the rows
+// of an item are consecutive positions of one sequence within one chunk.  mix_t: float32 [H][H], the
+// mixing matrix transposed (mix_t[g][h] multiplies head g's raw score into head h's), or null.
+HFEE_API int hfee_attention_mix_bf16(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
+                                     const int* items, int count, const int* block_tables, int bt_stride, int kv_heads,
+                                     int page_size, float scale, const float* mix_t, int chunk, int sink_mode,
+                                     const float* sinks, hipStream_t stream) {
+  HFEE_REQUIRE(count >= 0, "attention_mix_bf16: bad item count");
+  if (count == 0) return 0;
+  HFEE_REQUIRE(kv_heads > 0 && H % kv_heads == 0, "attention_mix_bf16: %d heads are not a multiple of %d kv heads", H, kv_heads);
+  HFEE_REQUIRE(chunk >= 0 && sink_mode >= 0 && sink_mode <= 2 && (sink_mode != 2 || sinks != nullptr),
+               "attention_mix_bf16: bad chunk or sink");
+  HFEE_REQUIRE(ldq >= (int64_t)H * D && ld_out >= (int64_t)H * D && ldq % 8 == 0 && ld_out % 4 == 0 &&
+               (uintptr_t)q % 16 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)cache % 16 == 0,
+               "attention_mix_bf16: q and out rows too short or not aligned");
+  KvLayout lay;
+  if (make_kv_layout(&lay, kv_heads, D, D, page_size)) return 1;
+  mix_attend_bf16_kernel<<<count, WAVES * 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache,
+                                                         lay, items, block_tables, bt_stride, scale, mix_t, chunk, sink_mode, sinks);
+  HFEE_CHECK_LAUNCH("attention_mix_bf16");
+  return 0;
+}

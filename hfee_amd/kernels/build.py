@@ -5,7 +5,9 @@ Two kinds of library:
   * `attention_bf16_hd<N>`: the matrix-core attention kernels, compiled for one head
     size each, on demand (a model compiles only the head size it has);
   * `attention_kv_bf16_k<Dk>_v<Dv>`: the matrix-core attention for keys and values of
-    different sizes, compiled per pair of sizes, on demand.
+    different sizes, compiled per pair of sizes, on demand;
+  * `attention_mix_bf16_h<H>_d<D>`: the matrix-core attention whose heads' scores are mixed,
+    compiled per number of heads and head size, on demand.
 Libraries are built in-tree (hfee_amd/_lib); if that folder cannot be written, in a
 per-user folder under the system's temporary directory; $HFEE_BUILD_DIR, if set, comes
 before both.  A library is rebuilt when its sources or flags no longer match the stamp
@@ -39,6 +41,16 @@ ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
 ATTENTION_KV_SOURCE = "attention_kv_bf16.hip"      # compiled per (key size, value size)
 ATTENTION_KV_MOST = (1024, 512)
+ATTENTION_MIX_SOURCE = "attention_mix_bf16.hip"    # compiled per (heads, head size)
+# the pairs that `build_all` compiles: those of the tests and of bench.py's comparison
+ATTENTION_MIX_SIZES = ((4, 32), (8, 32), (8, 64), (16, 128), (32, 128))
+
+
+def attention_mix_fits(heads: int, dim: int) -> bool:
+    """Whether the matrix-core kernels of attention with mixed heads take these sizes: heads in fours, head
+    sizes in multiples of 32, and what a wave keeps in registers (a quarter of the heads' queries and
+    outputs) within their number."""
+    return heads % 4 == 0 and dim % 32 == 0 and 4 <= heads <= 64 and heads // 4 * dim <= 1024
 # the pairs that `build_all` compiles: those of the tests and of bench.py's comparison (a model with
 # other sizes compiles its own at first use)
 ATTENTION_KV_SIZES = ((32, 16), (64, 32), (96, 64), (48, 32), (16, 48), (112, 96), (64, 64), (160, 128), (128, 128), (576, 512))
@@ -115,6 +127,14 @@ def library_spec(name: str):
             raise BuildError(f"the attention kernels for keys and values of different sizes take multiples of 16 up to "
                              f"{ATTENTION_KV_MOST}, not ({dk}, {dv})")
         return [ATTENTION_KV_SOURCE], [f"-DHFEE_DK={dk}", f"-DHFEE_DV={dv}"]
+    if name.startswith("attention_mix_bf16_h"):
+        try:
+            heads, dim = (int(n) for n in name[len("attention_mix_bf16_h"):].split("_d"))
+        except ValueError:
+            raise BuildError(f"unknown kernel library {name!r}") from None
+        if not attention_mix_fits(heads, dim):
+            raise BuildError(f"the matrix-core attention with mixed heads does not take {heads} heads of {dim}")
+        return [ATTENTION_MIX_SOURCE], [f"-DHFEE_MIX_HEADS={heads}", f"-DHFEE_MIX_DIM={dim}"]
     raise BuildError(f"unknown kernel library {name!r}")
 
 
@@ -188,12 +208,13 @@ def build_library(name: str, force: bool = False) -> str:
     return so
 
 
-def build_all(head_dims=HEAD_DIMS, force: bool = True, kv_sizes=ATTENTION_KV_SIZES) -> list:
+def build_all(head_dims=HEAD_DIMS, force: bool = True, kv_sizes=ATTENTION_KV_SIZES, mix_sizes=ATTENTION_MIX_SIZES) -> list:
     """Compiles the core library, the attention library of every head size, and the attention
     libraries for keys and values of different sizes of the listed pairs."""
     out = [build_library("core", force=force)]
     # the attention libraries are independent: build them side by side
     names = [f"attention_bf16_hd{hd}" for hd in head_dims] + [f"attention_kv_bf16_k{dk}_v{dv}" for dk, dv in kv_sizes]
+    names += [f"attention_mix_bf16_h{h}_d{d}" for h, d in mix_sizes]
     errors = []
 
     def work(n):

@@ -74,6 +74,12 @@ _ATTENTION_KV_SIGNATURES = {
     "hfee_attention_kv_bf16": [P, L, P, L, P, P, I, I, P, I, I, I, I, F, P, P, L, I, P],
 }
 
+_ATTENTION_MIX_SIGNATURES = {
+    "hfee_attention_mix_bf16_heads": [],
+    "hfee_attention_mix_bf16_dim": [],
+    "hfee_attention_mix_bf16": [P, L, P, L, P, P, I, P, I, I, I, F, P, I, I, P, P],
+}
+
 _ATTENTION_SIGNATURES = {
     "hfee_attention_bf16_head_dim": [],
     "hfee_attention_bf16_run_tiles": [],
@@ -124,7 +130,8 @@ def load(name: str) -> Library:
             except build.BuildError as e:
                 raise KernelLibraryError(f"the HIP kernel library '{name}' is not available: {e}") from None
             sigs = (_CORE_SIGNATURES if name == "core" else
-                    _ATTENTION_KV_SIGNATURES if name.startswith("attention_kv_bf16") else _ATTENTION_SIGNATURES)
+                    _ATTENTION_KV_SIGNATURES if name.startswith("attention_kv_bf16") else
+                    _ATTENTION_MIX_SIGNATURES if name.startswith("attention_mix_bf16") else _ATTENTION_SIGNATURES)
             lib = _loaded[name] = Library(name, path, sigs)
         return lib
 
@@ -146,3 +153,10 @@ def attention_kv_bf16(dk: int, dv: int) -> Library:
         raise KernelError(f"the bfloat16 attention kernels for keys and values of different sizes take multiples "
                           f"of 16, not ({dk}, {dv})")
     return load(f"attention_kv_bf16_k{dk}_v{dv}")
+
+
+def attention_mix_bf16(heads: int, dim: int) -> Library:
+    """The matrix-core attention with mixed heads for this number of heads and head size."""
+    if not build.attention_mix_fits(heads, dim):
+        raise KernelError(f"the matrix-core attention with mixed heads does not take {heads} heads of {dim}")
+    return load(f"attention_mix_bf16_h{heads}_d{dim}")

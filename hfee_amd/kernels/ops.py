@@ -999,9 +999,9 @@ def layernorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: flo
 # --------------------------------- attention whose heads' scores are mixed, over keys that are the values
 
 def _mix_cache(cache_layer, kv_heads, dim, page_size, what):
-    _check(cache_layer.is_contiguous() and cache_layer.dim() == 4 and
-           tuple(cache_layer.shape[1:]) == (kv_heads, page_size, 2 * dim),
-           f"{what}: the cache layer must be [pages, kv_heads, page_size, 2 * dim]")
+    _check(cache_layer.is_contiguous() and cache_layer.dim() == 3 and
+           tuple(cache_layer.shape[1:]) == (kv_heads, page_size * 2 * dim),
+           f"{what}: the cache layer must be [pages, kv_heads, page_size * 2 * dim]")
 
 
 def _tables(block_tables, what):
@@ -1014,8 +1014,8 @@ def attention_mix_prepare(q, k, positions, token_segment, block_tables, cos, sin
     """q ([n, num_heads * dim], in place) and k ([n, kv_heads * dim]) rotated in their first 2 * half
     dims (cos/sin float32 [positions, half], pairs (i, i + half)) and then, with `norm`, divided by
     their root mean square over each head; the key as it is scored and the key as it was projected
-    go into the token's slot of `cache_layer` ([pages, kv_heads, page_size, 2 * dim]).  k None: only
-    q is made ready."""
+    go into the token's slot of `cache_layer` ([pages, kv_heads, page_size * 2 * dim]: the scored keys of a
+    (page, head) as [slot][dim], then the values transposed as [dim][slot]).  k None: only q is made ready."""
     _gpu(q, k, positions, cos, sin, cache_layer)
     some = q if q is not None else k
     _check(some is not None, "attention_mix_prepare: nothing to do")
@@ -1051,7 +1051,7 @@ def attention_mix(out, q, cache_layer, positions, token_segment, block_tables, n
     position 0) up to p; the heads' scores q . k * scale are mixed by `mix` (float32 [heads, heads],
     score_h = sum_g mix[h, g] score_g; None: not mixed); sink: None, "zero" (one more term exp(0) in
     the softmax's denominator) or a float32 tensor [heads] of learned scores; the values are the
-    second half of each cache slot."""
+    second half of each (page, head) of the cache."""
     _gpu(out, q, cache_layer, positions, token_segment, block_tables, mix)
     n, w, ldq = _rows2d(q, "attention_mix q")
     no, wo, ldo = _rows2d(out, "attention_mix out")
@@ -1076,6 +1076,48 @@ def attention_mix(out, q, cache_layer, positions, token_segment, block_tables, n
     lib.core().call("hfee_attention_mix", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _dt(q), _ptr(positions),
                     _ptr(token_segment), _ptr(block_tables), block_tables.stride(0), num_heads, kv_heads, dim, page_size,
                     float(scale), _ptr(mix), int(chunk), mode, _ptr(sinks), n, _stream())
+
+
+def attention_mix_fits(num_heads: int, dim: int) -> bool:
+    """Whether the matrix-core kernels take these sizes (else: `attention_mix`)."""
+    from . import build
+    return build.attention_mix_fits(num_heads, dim)
+
+
+ATTENTION_MIX_ROWS = 16
+
+
+def attention_mix_bf16(out, q, cache_layer, items, block_tables, num_heads: int, kv_heads: int, dim: int, page_size: int,
+                       scale: float, mix_t=None, chunk: int = 0, sink=None):
+    """`attention_mix` on the matrix cores, bfloat16.  items: int32 [count, 4] on the device (first row,
+    rows (1 to 16), first position, block-table row), the rows of an item consecutive positions of one
+    sequence within one chunk; mix_t: the mixing matrix transposed, float32 [heads, heads]
+    (score_h = sum_g mix_t[g, h] score_g), or None."""
+    _gpu(out, q, cache_layer, items, block_tables, mix_t)
+    n, w, ldq = _rows2d(q, "attention_mix q")
+    no, wo, ldo = _rows2d(out, "attention_mix out")
+    _check(no == n and w == num_heads * dim and wo == num_heads * dim, "attention_mix: q/out shape")
+    _check(q.dtype == out.dtype == cache_layer.dtype == torch.bfloat16, "attention_mix: bfloat16 tensors expected")
+    _mix_cache(cache_layer, kv_heads, dim, page_size, "attention_mix")
+    _check(items.dtype == torch.int32 and items.dim() == 2 and items.shape[1] == 4 and items.is_contiguous(),
+           "attention_mix: items must be [count, 4] int32")
+    _tables(block_tables, "attention_mix")
+    if mix_t is not None:
+        _check(mix_t.dtype == torch.float32 and mix_t.is_contiguous() and tuple(mix_t.shape) == (num_heads, num_heads),
+               "attention_mix: mix_t must be float32 [heads, heads]")
+    sinks, mode = None, 0
+    if isinstance(sink, str):
+        _check(sink == "zero", "attention_mix: sink is None, 'zero' or a tensor")
+        mode = 1
+    elif sink is not None:
+        _gpu(sink)
+        _check(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == num_heads,
+               "attention_mix: sinks must be float32 [heads]")
+        sinks, mode = sink, 2
+    lib.attention_mix_bf16(num_heads, dim).call(
+        "hfee_attention_mix_bf16", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(items), items.shape[0],
+        _ptr(block_tables), block_tables.stride(0), kv_heads, page_size, float(scale), _ptr(mix_t), int(chunk), mode,
+        _ptr(sinks), _stream())
 
 
 # ------------------------------------------------ mixers with a state of fixed size a request

@@ -10,13 +10,16 @@ softmax are s_h = sum_g T[h, g] raw_g, T a learned [H, H] tensor.  Position i se
 the sequence.  `sink`: None, "zero" (the softmax's denominator holds one more term exp(0) that has no
 value) or "learned" (one score a head, a tensor).
 
-The cache layer keeps, for a token and key head, the key as it is scored and then the key as it was
+The cache layer keeps, for a token and key head, the key as it is scored and the key as it was
 projected; prompt portions and single tokens read both from there with the same kernel, in tiles of
-keys counted from the chunk's start, so that a token's result does not depend on how its sequence was
-cut into steps.
+keys whose place depends on positions only, so that a token's result does not depend on how its
+sequence was cut into steps.  In bfloat16, with heads in fours and head sizes in multiples of 32, the
+matrix-core kernel runs (rows of a sequence in items of up to 16 that do not cross a chunk's edge);
+any other size, and float32, goes through the plain kernel.
 """
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..config.specs import CacheNeed, MixerSpec
@@ -25,7 +28,7 @@ from ..weights.spec import TensorSpec
 from .base import LazyNorm, Mixer, lookup, register_mixer
 from .kv_attention import product, tiles_of
 
-_LAYOUT = "by key head and slot: the key as scored, then the key as projected"
+_LAYOUT = "by key head: the keys as scored by slot, then the keys as projected by dimension"
 
 
 @register_mixer("mixed_attention")
@@ -61,6 +64,8 @@ class MixedAttention(Mixer):
         defaults = dict(q="q_proj.weight", k="k_proj.weight", o="o_proj.weight", head_mix="head_mix", sink="sinks")
         self.names = {role: prefix + given.get(role, default) for role, default in defaults.items()}
         self.q_width, self.k_width = self.num_heads * self.dim, self.kv_heads * self.dim
+        self.matrix = dtype == torch.bfloat16 and ops.attention_mix_fits(self.num_heads, self.dim) and self.hidden % 8 == 0
+        self.items_key = f"mixed_attention.items.{self.chunk}"
 
     def tensor_specs(self):
         n, H = self.names, self.num_heads
@@ -77,6 +82,7 @@ class MixedAttention(Mixer):
         self.w_qk = torch.cat([tensors.pop(n["q"]), tensors.pop(n["k"])], dim=0).contiguous()
         self.w_o = tensors.pop(n["o"]).contiguous()
         self.mix = tensors.pop(n["head_mix"]).to(torch.float32).contiguous() if self.head_mix else None
+        self.mix_t = self.mix.t().contiguous() if self.mix is not None else None
         self.sinks = tensors.pop(n["sink"]).to(torch.float32).contiguous() if self.sink == "learned" else None
         self.w_qk_tiles, self.w_o_tiles = tiles_of(self.dtype, self.w_qk, self.w_o)
 
@@ -91,10 +97,27 @@ class MixedAttention(Mixer):
         if self.position is not None:
             self.position.prepare(info.num_positions, info.device)
 
+    def plan(self, plan):
+        """The step's rows in items of up to 16 that stay within a chunk (once a step and chunk size,
+        whichever layers ask): first row, rows, first position, block-table row."""
+        if not self.matrix or self.items_key in plan.arrays:
+            return
+        items = []
+        for s, seg in enumerate(plan.segments):
+            off = 0
+            while off < seg.length:
+                p = seg.start + off
+                room = min(ops.ATTENTION_MIX_ROWS, seg.length - off)
+                if self.chunk:
+                    room = min(room, self.chunk - p % self.chunk)
+                items.append((seg.row0 + off, room, p, s))
+                off += room
+        plan.add(self.items_key, np.asarray(items, dtype=np.int32).reshape(-1, 4))
+
     def forward_add(self, ctx, x, h, cache_layer: int, writes_cache: bool):
         hn = h.tensor() if isinstance(h, LazyNorm) else h
         H, G, D = self.num_heads, self.kv_heads, self.dim
-        cache = ctx.storage.layer(cache_layer, (G, ctx.page_size, 2 * D))
+        cache = ctx.storage.layer(cache_layer, (G, ctx.page_size * 2 * D))
         tables = ctx.block_tables[ctx.storage.group_of(cache_layer)]
         pos = self.position
         cos, sin = (pos.cos, pos.sin) if pos else (None, None)
@@ -109,6 +132,11 @@ class MixedAttention(Mixer):
         ops.attention_mix_prepare(q, k, ctx.positions, ctx.token_segment, tables, cos, sin, cache, H, G, D, ctx.page_size,
                                   ctx.max_position, norm=self.qk_norm is not None, eps=self.norm_eps)
         att = ctx.rows("mixed_attention.out", self.q_width)
-        ops.attention_mix(att, q, cache, ctx.positions, ctx.token_segment, tables, H, G, D, ctx.page_size, self.scale,
-                          mix=self.mix, chunk=self.chunk, sink="zero" if self.sink == "zero" else self.sinks)
+        sink = "zero" if self.sink == "zero" else self.sinks
+        if self.matrix:
+            ops.attention_mix_bf16(att, q, cache, ctx.extra[self.items_key], tables, H, G, D, ctx.page_size, self.scale,
+                                   mix_t=self.mix_t, chunk=self.chunk, sink=sink)
+        else:
+            ops.attention_mix(att, q, cache, ctx.positions, ctx.token_segment, tables, H, G, D, ctx.page_size, self.scale,
+                              mix=self.mix, chunk=self.chunk, sink=sink)
         product(ctx, x, att, self.w_o, self.w_o_tiles, add=True)

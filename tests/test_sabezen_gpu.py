@@ -122,7 +122,7 @@ def test_mixed_attention_kernels_with_a_key_that_stands_out(dtype, chunk, H, G, 
     got = torch.zeros(T, H * D, dtype=dt, device="cuda")
     cuts = [0, 37, 39, 100, 140] + list(range(141, T + 1))
     pos_all, seg_all, tables, pages = _paged([np.arange(T)], page, seed=1)
-    cache = torch.full((pages, G, page, 2 * D), float("nan"), dtype=dt, device="cuda")
+    cache = torch.full((pages, G, page * 2 * D), float("nan"), dtype=dt, device="cuda")
     for lo, hi in zip(cuts[:-1], cuts[1:]):
         qs, ks = q[lo:hi].reshape(hi - lo, -1).cuda().contiguous(), k[lo:hi].reshape(hi - lo, -1).cuda().contiguous()
         pos, seg = pos_all[lo:hi].contiguous(), seg_all[lo:hi].contiguous()
@@ -134,6 +134,79 @@ def test_mixed_attention_kernels_with_a_key_that_stands_out(dtype, chunk, H, G, 
     assert su.rel(got.double().cpu(), want) < tol
     for t in (last, last - 1, first, min(first + 1, last)):
         assert su.rel(got[t].double().cpu(), want[t]) < tol, f"token {t}"
+
+
+@pytest.mark.parametrize("chunk,H,G,D,half", [(24, 4, 2, 32, 8), (70, 8, 2, 64, 16), (0, 4, 4, 32, 0), (16, 8, 8, 32, 16)])
+def test_mixed_attention_on_the_matrix_cores(chunk, H, G, D, half):
+    """The matrix-core kernel against the plain mixer in float64 and against the plain kernel, with keys
+    that stand out at the chunk's first and last place and just outside it; the sequence comes in
+    portions whose items end at every chunk's edge, then token by token, beside a second sequence."""
+    from hfee_amd.kernels import ops
+    from hfee_amd.parts.rotary import rope_frequencies
+    T, page = 150, 16
+    g = torch.Generator().manual_seed(chunk + H)
+    size = chunk or T
+    q = torch.randn(2, T, H, D, generator=g)
+    k = torch.randn(2, T, G, D, generator=g)
+    last = T - 1
+    first = last // size * size
+    for j in (first, max(first - 1, 0), min(first + 1, last), last, 2):
+        k[:, j] *= 3.0
+    q[0, last] = k[0, first].repeat_interleave(H // G, dim=0) * 1.5 + q[0, last] * 0.1
+    if first > 0:
+        q[0, last - 1] = k[0, first - 1].repeat_interleave(H // G, dim=0) * 1.5
+    q, k = q.bfloat16(), k.bfloat16()
+    talk = torch.eye(H) + torch.randn(H, H, generator=g) * 0.3
+    m = {"heads": H, "kv_heads": G, "dim": D, "scale": 0.3, "mask": {"size": size}, "rot": {"dims": 2 * half, "base": 100.0}}
+    hidden = (H + G) * D
+    w = {"m.q": torch.eye(hidden)[:H * D].double(), "m.k": torch.eye(hidden)[H * D:].double(), "m.talk": talk.double(),
+         "m.o": torch.eye(H * D).double()}
+    want = [ps.chunked_talking_attention(torch.cat([q[s].reshape(T, -1), k[s].reshape(T, -1)], dim=1).double(), w, "m.", m, 1e-6)
+            for s in range(2)]
+    inv = rope_frequencies(2 * half, 100.0) if half else np.zeros(0)
+    ang = np.arange(T)[:, None] * inv[None, :]
+    cos, sin = (dev(np.cos(ang), torch.float32), dev(np.sin(ang), torch.float32)) if half else (None, None)
+    _, _, tables, pages = _paged([np.arange(T), np.arange(T)], page, seed=2)
+    cache = torch.zeros((pages, G, page * 2 * D), dtype=torch.bfloat16, device="cuda")
+    got = torch.zeros(2, T, H * D, dtype=torch.bfloat16, device="cuda")
+    plain = torch.zeros(2, T, H * D, dtype=torch.bfloat16, device="cuda")
+    fed = [0, 0]
+    steps = [(37, 5), (2, 60), (61, 0), (40, 45), (0, 30)] + [(1, 1)] * 10
+    for sizes in steps:
+        segs = [(s, n) for s, n in enumerate(sizes) if n]
+        pos = np.concatenate([np.arange(fed[s], fed[s] + n) for s, n in segs])
+        seg = np.concatenate([np.full(n, s) for s, n in segs])        # (the block table's row is the sequence)
+        qs = torch.cat([q[s, fed[s]:fed[s] + n].reshape(n, -1) for s, n in segs]).cuda().contiguous()
+        ks = torch.cat([k[s, fed[s]:fed[s] + n].reshape(n, -1) for s, n in segs]).cuda().contiguous()
+        ops.attention_mix_prepare(qs, ks, i32(pos), i32(seg), tables, cos, sin, cache, H, G, D, page, int(pos.max()),
+                                  norm=True, eps=1e-6)
+        items, row = [], 0
+        for s, n in segs:
+            off = 0
+            while off < n:
+                p = fed[s] + off
+                room = min(16, n - off, (chunk - p % chunk) if chunk else 16)
+                items.append((row + off, room, p, s))
+                off += room
+            row += n
+        out = torch.zeros(len(pos), H * D, dtype=torch.bfloat16, device="cuda")
+        ops.attention_mix_bf16(out, qs, cache, i32(np.asarray(items).reshape(-1, 4)), tables, H, G, D, page, 0.3,
+                               mix_t=talk.t().contiguous().cuda(), chunk=chunk, sink="zero")
+        ref = torch.zeros_like(out)
+        ops.attention_mix(ref, qs, cache, i32(pos), i32(seg), tables, H, G, D, page, 0.3, mix=talk.cuda(), chunk=chunk, sink="zero")
+        row = 0
+        for s, n in segs:
+            got[s, fed[s]:fed[s] + n] = out[row:row + n]
+            plain[s, fed[s]:fed[s] + n] = ref[row:row + n]
+            row += n
+            fed[s] += n
+    assert fed == [T, T]
+    for s in range(2):
+        assert su.rel(plain[s].double().cpu(), want[s]) < 3e-2
+        assert su.rel(got[s].double().cpu(), want[s]) < 3e-2
+        assert su.rel(got[s].double().cpu(), plain[s].double().cpu()) < 2e-2
+        for t in (last, last - 1, first, min(first + 1, last), 0, 1, 15, 16, 17):
+            assert su.rel(got[s, t].double().cpu(), want[s][t]) < 3e-2, f"sequence {s} token {t}"
 
 
 @pytest.mark.parametrize("rule", ["delta", "decay_add"])
