@@ -16,7 +16,10 @@
 //      four lanes of a row; the weights rounded to bfloat16 are, as they lie, the second operand of
 //   4. v_mfma_f32_16x16x16_bf16 with four keys of a value column (8 bytes of the page) as the first:
 //      out[head][16 dims][row] a register block.
-// A single token is an item of one row.
+// A single token is an item of one row.  Where a step has few items, the key tiles of an item are shared
+// out over several workgroups (`splits`): each leaves its running maximum, its sum and its unscaled
+// output in float32, and a second kernel joins them in the order of the splits; the sink belongs to the
+// first split.
 #include "attention_kv.h"
 
 using namespace hfee;
@@ -49,7 +52,8 @@ union Operand4 {
 __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
     bf16_t* __restrict__ out, int64_t ld_out, const bf16_t* __restrict__ q, int64_t ldq, const bf16_t* __restrict__ cache,
     KvLayout lay, const int* __restrict__ items, const int* __restrict__ block_tables, int bt_stride, float scale,
-    const float* __restrict__ mix_t, int chunk, int sink_mode, const float* __restrict__ sinks) {
+    const float* __restrict__ mix_t, int chunk, int sink_mode, const float* __restrict__ sinks, int splits,
+    float* __restrict__ partial_ml, float* __restrict__ partial_o) {
   __shared__ float raw[H][ROWS][KEYS];
   const int4 item = reinterpret_cast<const int4*>(items)[blockIdx.x];
   const int row0 = item.x, rows = item.y, p0 = item.z;
@@ -67,17 +71,23 @@ __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
     for (int ks = 0; ks < KS; ++ks)
       qop[hh][ks].u = *reinterpret_cast<const u32x4*>(q + (int64_t)(row0 + my_row) * ldq + (wave * HW + hh) * D + ks * 32 + kq * 8);
 
+  // this workgroup's share of the item's key tiles
+  const int tile0 = first / KEYS, tiles = last / KEYS - tile0 + 1, share = (tiles + splits - 1) / splits;
+  const int split = blockIdx.y;
+  const int j_begin = (tile0 + split * share) * KEYS, j_end = min(tile0 + tiles, tile0 + (split + 1) * share) * KEYS;
+  const int sinking = split == 0 ? sink_mode : 0;
+
   f32x4 o[HW][DB];
   float m[HW], l[HW];
 #pragma unroll
   for (int hh = 0; hh < HW; ++hh) {
-    m[hh] = sink_mode == 0 ? -INFINITY : sink_mode == 1 ? 0.f : sinks[wave * HW + hh];
-    l[hh] = sink_mode == 0 ? 0.f : 1.f;
+    m[hh] = sinking == 0 ? -INFINITY : sinking == 1 ? 0.f : sinks[wave * HW + hh];
+    l[hh] = sinking == 0 ? 0.f : 1.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db) o[hh][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int j0 = first & ~(KEYS - 1); j0 <= last; j0 += KEYS) {
+  for (int j0 = j_begin; j0 < j_end; j0 += KEYS) {
     const int page = bt[j0 >> lay.page_shift], slot0 = j0 & (lay.page_size - 1);
     // 1. raw scores of the wave's heads
 #pragma unroll
@@ -154,6 +164,21 @@ __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
     }
   }
   // register i of lane l: dim 16 db + 4 (l / 16) + i of row l % 16
+  if (splits > 1) {
+    if (r16 < rows) {
+#pragma unroll
+      for (int hh = 0; hh < HW; ++hh) {
+        const int64_t at = (((int64_t)blockIdx.x * splits + split) * H + wave * HW + hh) * ROWS + r16;
+        if (kq == 0) {
+          partial_ml[2 * at] = m[hh];
+          partial_ml[2 * at + 1] = l[hh];
+        }
+#pragma unroll
+        for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(partial_o + at * D + db * 16 + kq * 4) = o[hh][db];
+      }
+    }
+    return;
+  }
   if (r16 < rows) {
 #pragma unroll
     for (int hh = 0; hh < HW; ++hh) {
@@ -169,6 +194,29 @@ __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
   }
 }
 
+// grid (items, heads): out[row][head] = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M), the splits in their order.
+__global__ __launch_bounds__(256) void mix_join_kernel(bf16_t* __restrict__ out, int64_t ld_out, const int* __restrict__ items,
+                                                       int splits, const float* __restrict__ partial_ml,
+                                                       const float* __restrict__ partial_o) {
+  const int4 item = reinterpret_cast<const int4*>(items)[blockIdx.x];
+  const int row0 = item.x, rows = item.y, h = blockIdx.y;
+  for (int e = threadIdx.x; e < rows * D; e += blockDim.x) {
+    const int r = e / D, d = e - r * D;
+    float top = -INFINITY;
+    for (int s = 0; s < splits; ++s) top = fmaxf(top, partial_ml[2 * ((((int64_t)blockIdx.x * splits + s) * H + h) * ROWS + r)]);
+    float sum = 0.f, value = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const int64_t at = (((int64_t)blockIdx.x * splits + s) * H + h) * ROWS + r;
+      const float ms = partial_ml[2 * at];
+      if (ms == -INFINITY) continue;                      // (a share in which the row saw nothing)
+      const float w = expf(ms - top);
+      sum = fmaf(partial_ml[2 * at + 1], w, sum);
+      value = fmaf(partial_o[at * D + d], w, value);
+    }
+    out[(int64_t)(row0 + r) * ld_out + h * D + d] = float_to_bf16(value / sum);
+  }
+}
+
 }  // namespace
 
 HFEE_DEFINE_LAST_ERROR
@@ -179,10 +227,12 @@ HFEE_API int hfee_attention_mix_bf16_dim() { return D; }
 // items: int32 [count][4] on the device: first row, rows (1..16), first position, block-table row; the rows
 // of an item are consecutive positions of one sequence within one chunk.  mix_t: float32 [H][H], the
 // mixing matrix transposed (mix_t[g][h] multiplies head g's raw score into head h's), or null.
+// splits > 1: every item's key tiles over so many workgroups; partial: count * splits * H * 16 * (D + 2) float32.
 HFEE_API int hfee_attention_mix_bf16(void* out, int64_t ld_out, const void* q, int64_t ldq, const void* cache,
                                      const int* items, int count, const int* block_tables, int bt_stride, int kv_heads,
                                      int page_size, float scale, const float* mix_t, int chunk, int sink_mode,
-                                     const float* sinks, hipStream_t stream) {
+                                     const float* sinks, int splits, float* partial, int64_t partial_floats,
+                                     hipStream_t stream) {
   HFEE_REQUIRE(count >= 0, "attention_mix_bf16: bad item count");
   if (count == 0) return 0;
   HFEE_REQUIRE(kv_heads > 0 && H % kv_heads == 0, "attention_mix_bf16: %d heads are not a multiple of %d kv heads", H, kv_heads);
@@ -191,10 +241,21 @@ HFEE_API int hfee_attention_mix_bf16(void* out, int64_t ld_out, const void* q, i
   HFEE_REQUIRE(ldq >= (int64_t)H * D && ld_out >= (int64_t)H * D && ldq % 8 == 0 && ld_out % 4 == 0 &&
                (uintptr_t)q % 16 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)cache % 16 == 0,
                "attention_mix_bf16: q and out rows too short or not aligned");
+  HFEE_REQUIRE(splits >= 1 && splits <= 65535, "attention_mix_bf16: 1 to 65535 splits");
+  const int64_t places = (int64_t)count * splits * H * ROWS;
+  HFEE_REQUIRE(splits == 1 || (partial != nullptr && partial_floats >= places * (D + 2) && (uintptr_t)partial % 16 == 0),
+               "attention_mix_bf16: the splits need %lld float32 of scratch", (long long)(places * (D + 2)));
   KvLayout lay;
   if (make_kv_layout(&lay, kv_heads, D, D, page_size)) return 1;
-  mix_attend_bf16_kernel<<<count, WAVES * 64, 0, stream>>>((bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache,
-                                                         lay, items, block_tables, bt_stride, scale, mix_t, chunk, sink_mode, sinks);
+  float* partial_o = partial;                               // [places][D], then [places][2]
+  float* partial_ml = partial != nullptr ? partial + places * D : nullptr;
+  mix_attend_bf16_kernel<<<dim3(count, splits), WAVES * 64, 0, stream>>>(
+      (bf16_t*)out, ld_out, (const bf16_t*)q, ldq, (const bf16_t*)cache, lay, items, block_tables, bt_stride, scale, mix_t, chunk,
+      sink_mode, sinks, splits, partial_ml, partial_o);
   HFEE_CHECK_LAUNCH("attention_mix_bf16");
+  if (splits > 1) {
+    mix_join_kernel<<<dim3(count, H), 256, 0, stream>>>((bf16_t*)out, ld_out, items, splits, partial_ml, partial_o);
+    HFEE_CHECK_LAUNCH("attention_mix_join");
+  }
   return 0;
 }

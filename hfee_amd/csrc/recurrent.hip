@@ -10,8 +10,8 @@
 // `linear_scan` walks the tokens that a step brings for a request one after the other, from the
 // state that the steps before left in the request's slot, and leaves the new state there: a
 // portion of a prompt and a single token are the same kernel, and a token's result does not
-// depend on where its prompt was cut.  A wave owns four columns of S, a lane every sixteenth row of one
-// of them; the sixteen lanes of a column add their parts up in a fixed order.  In memory the state of a
+// depend on where its prompt was cut.  A wave owns four columns of S, a lane a sixteenth of the rows of
+// one of them; the sixteen lanes of a column add their parts up in a fixed order.  In memory the state of a
 // head lies as [blocks of four columns][D][4] (values that are no multiple of four are filled up).
 //
 // Around it, each in float32 whatever the engine's dtype:
@@ -101,38 +101,58 @@ __global__ __launch_bounds__(256) void scan_gate_kernel(float* __restrict__ out,
   out[t * ldo + c] = r;
 }
 
-// grid (column blocks of 4, heads, segments), one wave: lane = 16 * column + part.  A lane owns the rows
-// d = 16 i + part (i < DPT) of its column of S, so that the sixteen lanes of a column hold sixteen
-// neighbouring rows and a load instruction of the wave covers 64 neighbouring floats of the state, which
-// lies in memory as [slot][head][column block][D][4].  The rows' products are added in two chains a
-// lane and then over the sixteen lanes of the column in a fixed tree.  What the next token needs is asked
-// for before the current one is worked on.
-constexpr int kScanParts = 16, kScanColumns = 4;
+// grid (blocks of 16 columns, heads, segments), four waves; a wave owns four columns of S, lane =
+// 16 * column + part, and a lane the rows d = DPT * part + i (i < DPT) of its column.  The state lies in
+// memory as [slot][head][blocks of four columns][D][4].  The sixteen lanes of a column add their parts
+// up in a fixed tree.  The keys, queries, decays, values and writing strengths of the next TB tokens are
+// asked for by the whole workgroup while it works on the current TB, and wait in LDS: the walk over the
+// tokens, which nothing can shorten, reads only LDS and registers.
+constexpr int kScanParts = 16, kScanColumns = 4, kScanWaves = 4;
 
 template <int DPT>
-struct ScanInputs {
-  float k[DPT], q[DPT], a[DPT], v, b;
+struct ScanShape {
+  static constexpr int DP = kScanParts * DPT;                       // rows of S, filled up
+  static constexpr int TB = DPT <= 8 ? 16 : DPT == 16 ? 8 : 4;      // tokens a block
+  static constexpr int WIDE = 3 * TB * DP;                          // k, q, a of a block
+  static constexpr int BUFFER = WIDE + TB * kScanWaves * kScanColumns + TB;
+  static constexpr int PER_THREAD = WIDE / (kScanWaves * 64);
 };
 
-template <int DPT, int RULE>
-__device__ __forceinline__ void scan_load(ScanInputs<DPT>& in, const float* __restrict__ q, int64_t ldq,
-                                          const float* __restrict__ k, int64_t ldk, const float* __restrict__ v, int64_t ldv,
-                                          const float* __restrict__ decay, int64_t ldd, const float* __restrict__ beta,
-                                          int64_t ldb, int t, int g, int h, int col, bool live, int part, int D, int V) {
-  const float* qt = q + (int64_t)t * ldq + (int64_t)g * D;
-  const float* kt = k + (int64_t)t * ldk + (int64_t)g * D;
-  const float* at = decay + (int64_t)t * ldd + (int64_t)h * D;
+// What a lane needs of one token, read from a block in LDS (sixteen bytes a read where a lane has four
+// rows or more).
+template <int DPT>
+struct ScanToken {
+  float k[DPT], q[DPT], a[DPT], v, b;
+  __device__ __forceinline__ void read(const float* buffer, int t, int d0, int column) {
+    typedef ScanShape<DPT> Sh;
+    typedef float f32x4_t __attribute__((ext_vector_type(4)));
+    const float* kt = buffer + t * Sh::DP + d0;
+    const float* qt = kt + Sh::TB * Sh::DP;
+    const float* at = qt + Sh::TB * Sh::DP;
+    if constexpr (DPT % 4 == 0) {
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) {
-    const int d = i * kScanParts + part;
-    const bool in_d = d < D;
-    in.k[i] = in_d ? kt[d] : 0.f;
-    in.q[i] = in_d ? qt[d] : 0.f;
-    in.a[i] = in_d ? at[d] : 0.f;
+      for (int i = 0; i < DPT; i += 4) {
+        const f32x4_t kv = *reinterpret_cast<const f32x4_t*>(kt + i), qv = *reinterpret_cast<const f32x4_t*>(qt + i),
+                      av = *reinterpret_cast<const f32x4_t*>(at + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          k[i + j] = kv[j];
+          q[i + j] = qv[j];
+          a[i + j] = av[j];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) {
+        k[i] = kt[i];
+        q[i] = qt[i];
+        a[i] = at[i];
+      }
+    }
+    v = buffer[Sh::WIDE + t * kScanWaves * kScanColumns + column];
+    b = buffer[Sh::WIDE + Sh::TB * kScanWaves * kScanColumns + t];
   }
-  in.v = live ? v[(int64_t)t * ldv + (int64_t)h * V + col] : 0.f;
-  in.b = RULE == 1 ? beta[(int64_t)t * ldb + h] : 1.f;
-}
+};
 
 // Over the sixteen lanes of a column, which are one row of the data-parallel primitives: neighbours in a
 // quad, the quads of a half, the halves.  Every step adds two numbers that both lanes of a pair hold the
@@ -151,55 +171,97 @@ __device__ __forceinline__ float column_sum(float x) {
 }
 
 template <int DPT, int RULE>
-__global__ __launch_bounds__(64) void linear_scan_kernel(
+__global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
     float* __restrict__ out, int64_t ldo, float* __restrict__ state, const float* __restrict__ q, int64_t ldq,
     const float* __restrict__ k, int64_t ldk, const float* __restrict__ v, int64_t ldv, const float* __restrict__ decay,
     int64_t ldd, const float* __restrict__ beta, int64_t ldb, const int* __restrict__ segment_rows,
     const int* __restrict__ segment_lengths, const int* __restrict__ segment_slots, int heads, int qk_heads, int D, int V) {
-  const int seg = blockIdx.z, h = blockIdx.y;
-  const int part = threadIdx.x & (kScanParts - 1), c = threadIdx.x >> 4;
-  const int col = blockIdx.x * kScanColumns + c;
+  typedef ScanShape<DPT> Sh;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int seg = blockIdx.z, h = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int part = lane & (kScanParts - 1), c = lane >> 4;
+  const int block = blockIdx.x * kScanWaves + wave;                 // of four columns
+  const int col = block * kScanColumns + c;
   const bool live = col < V;
   const int g = h / (heads / qk_heads);
   const int blocks = (V + kScanColumns - 1) / kScanColumns;
-  float* S = state + ((((int64_t)segment_slots[seg] * heads + h) * blocks + blockIdx.x) * D) * kScanColumns + c;
+  const int d0 = part * DPT;
+  float* S = state + ((((int64_t)segment_slots[seg] * heads + h) * blocks + (live ? block : 0)) * D) * kScanColumns + c;
   float s[DPT];
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) {
-    const int d = i * kScanParts + part;
-    s[i] = d < D ? S[(int64_t)d * kScanColumns] : 0.f;
-  }
+  for (int i = 0; i < DPT; ++i) s[i] = live && d0 + i < D ? S[(int64_t)(d0 + i) * kScanColumns] : 0.f;
   const int row0 = segment_rows[seg], len = segment_lengths[seg];
-  ScanInputs<DPT> now, next;
-  scan_load<DPT, RULE>(now, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, row0, g, h, col, live, part, D, V);
-  for (int t = row0; t < row0 + len; ++t) {
-    if (t + 1 < row0 + len)
-      scan_load<DPT, RULE>(next, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, t + 1, g, h, col, live, part, D, V);
-    float u = now.v;
-    if constexpr (RULE == 1) {
-      float d0 = 0.f, d1 = 0.f;
+
+  float wide[Sh::PER_THREAD], narrow = 0.f, strength = 0.f;
+  auto ask = [&](int first) {          // the block of tokens that begins at `first`, into registers
+#pragma unroll
+    for (int r = 0; r < Sh::PER_THREAD; ++r) {
+      const int e = tid + r * kScanWaves * 64;
+      const int which = e / (Sh::TB * Sh::DP), rest = e - which * (Sh::TB * Sh::DP);
+      const int t = rest / Sh::DP, d = rest - t * Sh::DP;
+      float x = 0.f;
+      if (first + t < len && d < D) {
+        const int64_t row = row0 + first + t;
+        x = which == 0 ? k[row * ldk + (int64_t)g * D + d] : which == 1 ? q[row * ldq + (int64_t)g * D + d]
+                                                                      : decay[row * ldd + (int64_t)h * D + d];
+      }
+      wide[r] = x;
+    }
+    {
+      const int t = tid / (kScanWaves * kScanColumns), cc = tid - t * (kScanWaves * kScanColumns);
+      const int column = blockIdx.x * kScanWaves * kScanColumns + cc;
+      narrow = t < Sh::TB && first + t < len && column < V ? v[(int64_t)(row0 + first + t) * ldv + (int64_t)h * V + column] : 0.f;
+    }
+    if (RULE == 1 && tid < Sh::TB) strength = first + tid < len ? beta[(int64_t)(row0 + first + tid) * ldb + h] : 0.f;
+  };
+  auto put = [&](float* buffer) {
+#pragma unroll
+    for (int r = 0; r < Sh::PER_THREAD; ++r) buffer[tid + r * kScanWaves * 64] = wide[r];
+    if (tid < Sh::TB * kScanWaves * kScanColumns) buffer[Sh::WIDE + tid] = narrow;
+    if (RULE == 1 && tid < Sh::TB) buffer[Sh::WIDE + Sh::TB * kScanWaves * kScanColumns + tid] = strength;
+  };
+
+  ask(0);
+  put(lds);
+  __syncthreads();
+  for (int first = 0, turn = 0; first < len; first += Sh::TB, turn ^= 1) {
+    const float* buffer = lds + turn * Sh::BUFFER;
+    const bool more = first + Sh::TB < len;
+    if (more) ask(first + Sh::TB);
+    const int count = min(Sh::TB, len - first);
+    ScanToken<DPT> now, next;
+    now.read(buffer, 0, d0, wave * kScanColumns + c);
+    for (int t = 0; t < count; ++t) {
+      if (t + 1 < count) next.read(buffer, t + 1, d0, wave * kScanColumns + c);      // (ahead of the sums that wait on one another)
+      float u = now.v;
+      if constexpr (RULE == 1) {
+        float p0 = 0.f, p1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < DPT; ++i) {
+          s[i] *= now.a[i];
+          if (i & 1) p1 = fmaf(s[i], now.k[i], p1); else p0 = fmaf(s[i], now.k[i], p0);
+        }
+        u = now.b * (now.v - column_sum(p0 + p1));
+      }
+      float o0 = 0.f, o1 = 0.f;
 #pragma unroll
       for (int i = 0; i < DPT; ++i) {
-        s[i] *= now.a[i];
-        if (i & 1) d1 = fmaf(s[i], now.k[i], d1); else d0 = fmaf(s[i], now.k[i], d0);
+        if constexpr (RULE == 1) s[i] = fmaf(now.k[i], u, s[i]);
+        else s[i] = fmaf(s[i], now.a[i], now.k[i] * u);
+        if (i & 1) o1 = fmaf(s[i], now.q[i], o1); else o0 = fmaf(s[i], now.q[i], o0);
       }
-      u = now.b * (now.v - column_sum(d0 + d1));
+      const float o = column_sum(o0 + o1);
+      if (live && part == 0) out[(int64_t)(row0 + first + t) * ldo + (int64_t)h * V + col] = o;
+      now = next;
     }
-    float o0 = 0.f, o1 = 0.f;
-#pragma unroll
-    for (int i = 0; i < DPT; ++i) {
-      if constexpr (RULE == 1) s[i] = fmaf(now.k[i], u, s[i]);
-      else s[i] = fmaf(s[i], now.a[i], now.k[i] * u);
-      if (i & 1) o1 = fmaf(s[i], now.q[i], o1); else o0 = fmaf(s[i], now.q[i], o0);
-    }
-    const float o = column_sum(o0 + o1);
-    if (live && part == 0) out[(int64_t)t * ldo + (int64_t)h * V + col] = o;
-    now = next;
+    if (more) put(lds + (turn ^ 1) * Sh::BUFFER);
+    __syncthreads();
   }
+  if (live) {
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) {
-    const int d = i * kScanParts + part;
-    if (d < D) S[(int64_t)d * kScanColumns] = s[i];
+    for (int i = 0; i < DPT; ++i)
+      if (d0 + i < D) S[(int64_t)(d0 + i) * kScanColumns] = s[i];
   }
 }
 
@@ -306,11 +368,11 @@ HFEE_API int hfee_linear_scan(float* out, int64_t ldo, float* state, const float
   HFEE_REQUIRE(rule == 0 || (rule == 1 && beta != nullptr), "linear_scan: rule 0, or rule 1 with its writing strengths");
   HFEE_REQUIRE(ldq >= (int64_t)qk_heads * dim && ldk >= (int64_t)qk_heads * dim && ldv >= (int64_t)heads * vdim &&
                ldd >= (int64_t)heads * dim && ldo >= (int64_t)heads * vdim, "linear_scan: rows too short");
-  dim3 grid((vdim + kScanColumns - 1) / kScanColumns, heads, segments);
-  HFEE_REQUIRE(grid.x <= 65535u * 32u, "linear_scan: values too wide");
+  const int columns = kScanWaves * kScanColumns;
+  dim3 grid((vdim + columns - 1) / columns, heads, segments);
   const int per = (dim + kScanParts - 1) / kScanParts;
 #define LAUNCH(DPT, RULE)                                                                                             \
-  linear_scan_kernel<DPT, RULE><<<grid, 64, 0, stream>>>(out, ldo, state, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, \
+  linear_scan_kernel<DPT, RULE><<<grid, kScanWaves * 64, 2 * ScanShape<DPT>::BUFFER * sizeof(float), stream>>>(out, ldo, state, q, ldq, k, ldk, v, ldv, decay, ldd, beta, ldb, \
       segment_rows, segment_lengths, segment_slots, heads, qk_heads, dim, vdim)
 #define PICK(RULE)                                                                                                    \
   if (per <= 1) LAUNCH(1, RULE); else if (per <= 2) LAUNCH(2, RULE); else if (per <= 4) LAUNCH(4, RULE);              \

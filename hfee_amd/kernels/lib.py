@@ -77,7 +77,7 @@ _ATTENTION_KV_SIGNATURES = {
 _ATTENTION_MIX_SIGNATURES = {
     "hfee_attention_mix_bf16_heads": [],
     "hfee_attention_mix_bf16_dim": [],
-    "hfee_attention_mix_bf16": [P, L, P, L, P, P, I, P, I, I, I, F, P, I, I, P, P],
+    "hfee_attention_mix_bf16": [P, L, P, L, P, P, I, P, I, I, I, F, P, I, I, P, I, P, L, P],
 }
 
 _ATTENTION_SIGNATURES = {

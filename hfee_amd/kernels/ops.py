@@ -1087,13 +1087,21 @@ def attention_mix_fits(num_heads: int, dim: int) -> bool:
 ATTENTION_MIX_ROWS = 16
 
 
+def attention_mix_partial_words(num_items: int, num_heads: int, dim: int, splits: int) -> int:
+    return num_items * splits * num_heads * ATTENTION_MIX_ROWS * (dim + 2) if splits > 1 else 0
+
+
 def attention_mix_bf16(out, q, cache_layer, items, block_tables, num_heads: int, kv_heads: int, dim: int, page_size: int,
-                       scale: float, mix_t=None, chunk: int = 0, sink=None):
+                       scale: float, mix_t=None, chunk: int = 0, sink=None, splits: int = 1, partial=None):
     """`attention_mix` on the matrix cores, bfloat16.  items: int32 [count, 4] on the device (first row,
     rows (1 to 16), first position, block-table row), the rows of an item consecutive positions of one
     sequence within one chunk; mix_t: the mixing matrix transposed, float32 [heads, heads]
-    (score_h = sum_g mix_t[g, h] score_g), or None."""
-    _gpu(out, q, cache_layer, items, block_tables, mix_t)
+    (score_h = sum_g mix_t[g, h] score_g), or None.  splits > 1: the key tiles of every item are shared out
+    over so many workgroups, which leave their parts in `partial` (float32, `attention_mix_partial_words`)
+    for a joining kernel."""
+    _gpu(out, q, cache_layer, items, block_tables, mix_t, partial)
+    if partial is not None:
+        _check(partial.dtype == torch.float32 and partial.is_contiguous(), "attention_mix: float32 partial buffer expected")
     n, w, ldq = _rows2d(q, "attention_mix q")
     no, wo, ldo = _rows2d(out, "attention_mix out")
     _check(no == n and w == num_heads * dim and wo == num_heads * dim, "attention_mix: q/out shape")
@@ -1117,7 +1125,7 @@ def attention_mix_bf16(out, q, cache_layer, items, block_tables, num_heads: int,
     lib.attention_mix_bf16(num_heads, dim).call(
         "hfee_attention_mix_bf16", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(items), items.shape[0],
         _ptr(block_tables), block_tables.stride(0), kv_heads, page_size, float(scale), _ptr(mix_t), int(chunk), mode,
-        _ptr(sinks), _stream())
+        _ptr(sinks), int(splits), _ptr(partial), 0 if partial is None else partial.numel(), _stream())
 
 
 # ------------------------------------------------ mixers with a state of fixed size a request

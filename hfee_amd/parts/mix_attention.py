@@ -28,6 +28,9 @@ from ..weights.spec import TensorSpec
 from .base import LazyNorm, Mixer, lookup, register_mixer
 from .kv_attention import product, tiles_of
 
+_WORKGROUPS_WANTED = 512        # items split their keys until about this many workgroups run
+_MOST_SPLITS = 8
+_PARTIAL_LIMIT = 64 << 20       # float32 words of the splits' parts
 _LAYOUT = "by key head: the keys as scored by slot, then the keys as projected by dimension"
 
 
@@ -134,8 +137,20 @@ class MixedAttention(Mixer):
         att = ctx.rows("mixed_attention.out", self.q_width)
         sink = "zero" if self.sink == "zero" else self.sinks
         if self.matrix:
-            ops.attention_mix_bf16(att, q, cache, ctx.extra[self.items_key], tables, H, G, D, ctx.page_size, self.scale,
-                                   mix_t=self.mix_t, chunk=self.chunk, sink=sink)
+            items = ctx.extra[self.items_key]
+            # the most key tiles an item can have: a chunk's, or the context's (under a captured graph the block
+            # table's whole width, so that a replay runs what was recorded)
+            span = self.chunk or ctx.host.get("graph.max_context", ctx.max_position + 1)
+            count = items.shape[0]
+            splits = max(1, min(-(-span // 16) // 4, _WORKGROUPS_WANTED // count, _MOST_SPLITS))
+            while splits > 1 and ops.attention_mix_partial_words(count, H, D, splits) > _PARTIAL_LIMIT:
+                splits -= 1
+            partial = None
+            if splits > 1:
+                partial = ctx.workspace.flat("mixed_attention.partial", ops.attention_mix_partial_words(count, H, D, splits),
+                                             torch.float32)
+            ops.attention_mix_bf16(att, q, cache, items, tables, H, G, D, ctx.page_size, self.scale, mix_t=self.mix_t,
+                                   chunk=self.chunk, sink=sink, splits=splits, partial=partial)
         else:
             ops.attention_mix(att, q, cache, ctx.positions, ctx.token_segment, tables, H, G, D, ctx.page_size, self.scale,
                               mix=self.mix, chunk=self.chunk, sink=sink)

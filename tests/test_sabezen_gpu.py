@@ -190,8 +190,11 @@ def test_mixed_attention_on_the_matrix_cores(chunk, H, G, D, half):
                 off += room
             row += n
         out = torch.zeros(len(pos), H * D, dtype=torch.bfloat16, device="cuda")
+        splits = 1 + len(pos) % 4                      # (the key tiles of an item over one to four workgroups)
+        partial = torch.full((ops.attention_mix_partial_words(len(items), H, D, splits),), float("nan"), device="cuda")
         ops.attention_mix_bf16(out, qs, cache, i32(np.asarray(items).reshape(-1, 4)), tables, H, G, D, page, 0.3,
-                               mix_t=talk.t().contiguous().cuda(), chunk=chunk, sink="zero")
+                               mix_t=talk.t().contiguous().cuda(), chunk=chunk, sink="zero", splits=splits,
+                               partial=partial if splits > 1 else None)
         ref = torch.zeros_like(out)
         ops.attention_mix(ref, qs, cache, i32(pos), i32(seg), tables, H, G, D, page, 0.3, mix=talk.cuda(), chunk=chunk, sink="zero")
         row = 0
