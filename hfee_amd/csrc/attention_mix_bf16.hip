@@ -3,8 +3,8 @@
 // multiple of 32).  What is computed is what attention_mix.hip computes (keys of the query's chunk up to
 // the query, scores of all heads mixed by a matrix, an optional sink, the keys as projected for values).
 //
-// A workgroup of four waves takes an item: up to 16 consecutive rows of one sequence that lie in one
-// chunk, and all heads, a wave H/4 of them.  Keys come in tiles of 16 that start at multiples of 16 of
+// A workgroup of four (or eight) waves takes an item: up to 16 consecutive rows of one sequence that lie in
+// one chunk, and all heads, a wave a quarter (an eighth) of them.  Keys come in tiles of 16 that start at multiples of 16 of
 // the sequence's positions (a tile lies in one page; keys before the chunk are masked), so what is added
 // in which order depends on positions only.  A tile's steps:
 //   1. raw scores: v_mfma_f32_16x16x32_bf16, the tile's keys as the first operand straight from the
@@ -31,8 +31,12 @@ using namespace hfee;
 namespace {
 
 constexpr int H = HFEE_MIX_HEADS, D = HFEE_MIX_DIM;
-constexpr int WAVES = 4, HW = H / WAVES, KS = D / 32, DB = D / 16, ROWS = 16, KEYS = 16;
-static_assert(H % WAVES == 0 && D % 32 == 0, "heads in fours, head sizes in multiples of 32");
+// (what a wave keeps in registers for all tiles, its heads' queries and outputs, is 3/8 of a register a
+// head and dim: four waves where that fits their 512 registers, eight waves of half as many heads and
+// 256 registers beyond)
+constexpr int WAVES = H / 4 * D > 512 ? 8 : 4;
+constexpr int HW = H / WAVES, KS = D / 32, DB = D / 16, ROWS = 16, KEYS = 16;
+static_assert(H % WAVES == 0 && D % 32 == 0 && HW * D <= 512, "heads in fours or eights, head sizes in multiples of 32");
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));

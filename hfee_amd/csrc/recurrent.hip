@@ -193,6 +193,39 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
   for (int i = 0; i < DPT; ++i) s[i] = live && d0 + i < D ? S[(int64_t)(d0 + i) * kScanColumns] : 0.f;
   const int row0 = segment_rows[seg], len = segment_lengths[seg];
 
+  if (len == 1) {      // a single token (every thread of the workgroup sees the same len): straight from memory
+    const int64_t row = row0;
+    float u = live ? v[row * ldv + (int64_t)h * V + col] : 0.f;
+    float kk[DPT], qq[DPT], aa[DPT];
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      const bool in = d0 + i < D;
+      kk[i] = in ? k[row * ldk + (int64_t)g * D + d0 + i] : 0.f;
+      qq[i] = in ? q[row * ldq + (int64_t)g * D + d0 + i] : 0.f;
+      aa[i] = in ? decay[row * ldd + (int64_t)h * D + d0 + i] : 0.f;
+    }
+    if constexpr (RULE == 1) {
+      float p0 = 0.f, p1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) {
+        s[i] *= aa[i];
+        if (i & 1) p1 = fmaf(s[i], kk[i], p1); else p0 = fmaf(s[i], kk[i], p0);
+      }
+      u = beta[row * ldb + h] * (u - column_sum(p0 + p1));
+    }
+    float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < DPT; ++i) {
+      if constexpr (RULE == 1) s[i] = fmaf(kk[i], u, s[i]);
+      else s[i] = fmaf(s[i], aa[i], kk[i] * u);
+      if (i & 1) o1 = fmaf(s[i], qq[i], o1); else o0 = fmaf(s[i], qq[i], o0);
+      if (live && d0 + i < D) S[(int64_t)(d0 + i) * kScanColumns] = s[i];
+    }
+    const float o = column_sum(o0 + o1);
+    if (live && part == 0) out[row * ldo + (int64_t)h * V + col] = o;
+    return;
+  }
+
   float wide[Sh::PER_THREAD], narrow = 0.f, strength = 0.f;
   auto ask = [&](int first) {          // the block of tokens that begins at `first`, into registers
 #pragma unroll

@@ -50,7 +50,10 @@ def attention_mix_fits(heads: int, dim: int) -> bool:
     """Whether the matrix-core kernels of attention with mixed heads take these sizes: heads in fours, head
     sizes in multiples of 32, and what a wave keeps in registers (a quarter of the heads' queries and
     outputs) within their number."""
-    return heads % 4 == 0 and dim % 32 == 0 and 4 <= heads <= 64 and heads // 4 * dim <= 1024
+    if heads % 4 or dim % 32 or not 4 <= heads <= 64:
+        return False
+    waves = 8 if heads // 4 * dim > 512 else 4
+    return heads % waves == 0 and heads // waves * dim <= 512
 # the pairs that `build_all` compiles: those of the tests and of bench.py's comparison (a model with
 # other sizes compiles its own at first use)
 ATTENTION_KV_SIZES = ((32, 16), (64, 32), (96, 64), (48, 32), (16, 48), (112, 96), (64, 64), (160, 128), (128, 128), (576, 512))
