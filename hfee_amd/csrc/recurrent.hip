@@ -12,7 +12,7 @@
 // portion of a prompt and a single token are the same kernel, and a token's result does not
 // depend on where its prompt was cut.  A wave owns four columns of S, a lane a sixteenth of the rows of
 // one of them; the sixteen lanes of a column add their parts up in a fixed order.  In memory the state of a
-// head lies as [blocks of four columns][D][4] (values that are no multiple of four are filled up).
+// head lies in blocks of four columns, each in the order in which a wave's lanes hold it.
 //
 // Around it, each in float32 whatever the engine's dtype:
 //   short_conv_silu     y_t = silu(sum_j taps[K-1-j] x_(t-j)) per channel, the K-1 inputs before the
@@ -102,8 +102,10 @@ __global__ __launch_bounds__(256) void scan_gate_kernel(float* __restrict__ out,
 }
 
 // grid (blocks of 16 columns, heads, segments), four waves; a wave owns four columns of S, lane =
-// 16 * column + part, and a lane the rows d = DPT * part + i (i < DPT) of its column.  The state lies in
-// memory as [slot][head][blocks of four columns][D][4].  The sixteen lanes of a column add their parts
+// 16 * column + part, and a lane the rows d = DPT * part + i (i < DPT) of its column (DPT = D / 16 filled up
+// to a power of two).  The state lies in memory as [slot][head][blocks of four columns][i][lane]: a wave's
+// load or store is 256 neighbouring bytes; rows at and beyond D and columns at and beyond V are zeros
+// that stay zeros.  The sixteen lanes of a column add their parts
 // up in a fixed tree.  The keys, queries, decays, values and writing strengths of the next TB tokens are
 // asked for by the whole workgroup while it works on the current TB, and wait in LDS: the walk over the
 // tokens, which nothing can shorten, reads only LDS and registers.
@@ -187,22 +189,42 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
   const int g = h / (heads / qk_heads);
   const int blocks = (V + kScanColumns - 1) / kScanColumns;
   const int d0 = part * DPT;
-  float* S = state + ((((int64_t)segment_slots[seg] * heads + h) * blocks + (live ? block : 0)) * D) * kScanColumns + c;
+  // (a wave whose four columns all lie beyond V works on the last block's numbers and stores nothing)
+  const bool mine = block < blocks;
+  float* S = state + (((int64_t)segment_slots[seg] * heads + h) * blocks + (mine ? block : blocks - 1)) * (DPT * 64) + lane;
   float s[DPT];
 #pragma unroll
-  for (int i = 0; i < DPT; ++i) s[i] = live && d0 + i < D ? S[(int64_t)(d0 + i) * kScanColumns] : 0.f;
+  for (int i = 0; i < DPT; ++i) s[i] = S[i * 64];
   const int row0 = segment_rows[seg], len = segment_lengths[seg];
 
   if (len == 1) {      // a single token (every thread of the workgroup sees the same len): straight from memory
     const int64_t row = row0;
     float u = live ? v[row * ldv + (int64_t)h * V + col] : 0.f;
     float kk[DPT], qq[DPT], aa[DPT];
+    const float* kp = k + row * ldk + (int64_t)g * D + d0;
+    const float* qp = q + row * ldq + (int64_t)g * D + d0;
+    const float* ap = decay + row * ldd + (int64_t)h * D + d0;
+    if (DPT % 4 == 0 && D == DPT * kScanParts && (((uintptr_t)kp | (uintptr_t)qp | (uintptr_t)ap) & 15) == 0) {
+      typedef float f32x4_t __attribute__((ext_vector_type(4)));      // (sixteen bytes a load where the rows allow)
 #pragma unroll
-    for (int i = 0; i < DPT; ++i) {
-      const bool in = d0 + i < D;
-      kk[i] = in ? k[row * ldk + (int64_t)g * D + d0 + i] : 0.f;
-      qq[i] = in ? q[row * ldq + (int64_t)g * D + d0 + i] : 0.f;
-      aa[i] = in ? decay[row * ldd + (int64_t)h * D + d0 + i] : 0.f;
+      for (int i = 0; i + 3 < DPT; i += 4) {
+        const f32x4_t kv = *reinterpret_cast<const f32x4_t*>(kp + i), qv = *reinterpret_cast<const f32x4_t*>(qp + i),
+                      av = *reinterpret_cast<const f32x4_t*>(ap + i);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          kk[i + j] = kv[j];
+          qq[i + j] = qv[j];
+          aa[i + j] = av[j];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < DPT; ++i) {
+        const bool in = d0 + i < D;
+        kk[i] = in ? kp[i] : 0.f;
+        qq[i] = in ? qp[i] : 0.f;
+        aa[i] = in ? ap[i] : 0.f;
+      }
     }
     if constexpr (RULE == 1) {
       float p0 = 0.f, p1 = 0.f;
@@ -219,7 +241,7 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
       if constexpr (RULE == 1) s[i] = fmaf(kk[i], u, s[i]);
       else s[i] = fmaf(s[i], aa[i], kk[i] * u);
       if (i & 1) o1 = fmaf(s[i], qq[i], o1); else o0 = fmaf(s[i], qq[i], o0);
-      if (live && d0 + i < D) S[(int64_t)(d0 + i) * kScanColumns] = s[i];
+        if (mine) S[i * 64] = s[i];
     }
     const float o = column_sum(o0 + o1);
     if (live && part == 0) out[row * ldo + (int64_t)h * V + col] = o;
@@ -291,10 +313,9 @@ __global__ __launch_bounds__(kScanWaves * 64) void linear_scan_kernel(
     if (more) put(lds + (turn ^ 1) * Sh::BUFFER);
     __syncthreads();
   }
-  if (live) {
+  if (mine) {
 #pragma unroll
-    for (int i = 0; i < DPT; ++i)
-      if (d0 + i < D) S[(int64_t)(d0 + i) * kScanColumns] = s[i];
+    for (int i = 0; i < DPT; ++i) S[i * 64] = s[i];
   }
 }
 

@@ -1201,18 +1201,24 @@ def scan_gate(out, z, kind: str, bias=None, per_head=None, head_width: int = 0, 
                     SCAN_GATES[kind], float(number), int(first_columns), n, w, _stream())
 
 
-SCAN_COLUMNS = 4
+SCAN_COLUMNS, SCAN_PARTS = 4, 16
+
+
+def _scan_rows_a_lane(dim: int) -> int:
+    per = (dim + SCAN_PARTS - 1) // SCAN_PARTS
+    return 1 << max(0, (per - 1).bit_length())
 
 
 def scan_state_shape(dim: int, vdim: int) -> tuple:
-    """How `linear_scan` keeps a head's matrix S [dim, vdim]: [blocks of four columns, dim, 4]."""
-    return ((vdim + SCAN_COLUMNS - 1) // SCAN_COLUMNS, dim, SCAN_COLUMNS)
+    """How `linear_scan` keeps a head's matrix S [dim, vdim]: blocks of four columns, each as the 64 lanes
+    of a wave hold it: [blocks, rows a lane, 4 columns, 16 parts], row d = rows a lane * part + i."""
+    return ((vdim + SCAN_COLUMNS - 1) // SCAN_COLUMNS, _scan_rows_a_lane(dim), SCAN_COLUMNS, SCAN_PARTS)
 
 
-def scan_state_matrix(state: torch.Tensor, vdim: int) -> torch.Tensor:
-    """[..., blocks, dim, 4] as `linear_scan` keeps it -> [..., dim, vdim]."""
-    s = state.transpose(-3, -2)
-    return s.reshape(*s.shape[:-2], -1)[..., :vdim]
+def scan_state_matrix(state: torch.Tensor, dim: int, vdim: int) -> torch.Tensor:
+    """[..., blocks, rows a lane, 4, 16] as `linear_scan` keeps it -> [..., dim, vdim]."""
+    s = state.permute(*range(state.dim() - 4), -1, -3, -4, -2)         # [..., part, i, block, column]
+    return s.reshape(*s.shape[:-4], s.shape[-4] * s.shape[-3], s.shape[-2] * s.shape[-1])[..., :dim, :vdim]
 
 
 def linear_scan(out, state, q, k, v, decay, beta, segment_rows, segment_lengths, segment_slots, heads: int,

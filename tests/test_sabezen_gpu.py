@@ -262,7 +262,7 @@ def test_linear_scan_in_portions(rule, H, G, D, V):
     assert fed == T
     for s in range(2):
         assert su.rel(got[s], want[s]) < 2e-5
-        assert su.rel(ops.scan_state_matrix(state[slots[s]], V).cpu(), torch.stack(final[s])) < 2e-5
+        assert su.rel(ops.scan_state_matrix(state[slots[s]], D, V).cpu(), torch.stack(final[s])) < 2e-5
     assert bool(torch.isnan(state[1]).all()) and float(state[2].abs().sum()) == 0.0
 
 
