@@ -29,8 +29,8 @@ class ChunkedAttentionConfig:
     dim: int
     vdim: int
     scale: float
-    chunk: int
-    rot: RotaryConfig
+    chunk: int                      # 0: no chunks
+    rot: Optional[RotaryConfig]
     type: str = "attention"
 
     @staticmethod
@@ -39,26 +39,35 @@ class ChunkedAttentionConfig:
         heads, dim = r.int("heads"), r.int("dim")
         kv_heads, vdim = r.int("kv_heads", heads), r.int("vdim", dim)
         scale = r.float("scale")
-        rot, mask = r.object("rot"), r.object("mask")
+        # (a layer whose entry names no mask sees every earlier position; one that names no rotation is not rotated)
+        rot, mask = r.object("rot", None), r.object("mask", None)
         r.require(not heads or not kv_heads or (heads > 0 and kv_heads > 0 and heads % kv_heads == 0),
                   f"{heads} heads are not a multiple of {kv_heads} kv_heads")
         _positive(r, dim=dim, vdim=vdim)
         r.require(dim is None or vdim == dim, f"the values are the keys: vdim {vdim} must equal dim {dim}")
         r.finish()
-        rm = KeyReader(mask, where + ".mask")
-        chunk = rm.int("size")
-        _positive(rm, size=chunk)
-        rm.finish()
-        rc = RotaryConfig.read(rot, where + ".rot")
-        if rc.scaling is not None:
-            raise ConfigError(f"{where}.rot: this design's rotation is not stretched")
-        if rc.dims > dim:
-            raise ConfigError(f"{where}: {rc.dims} rotated dims do not fit a head of {dim}")
+        chunk = 0
+        if mask is not None:
+            rm = KeyReader(mask, where + ".mask")
+            chunk = rm.int("size")
+            _positive(rm, size=chunk)
+            rm.finish()
+        rc = None
+        if rot is not None:
+            rc = RotaryConfig.read(rot, where + ".rot")
+            if rc.scaling is not None:
+                raise ConfigError(f"{where}.rot: this design's rotation is not stretched")
+            if rc.dims > dim:
+                raise ConfigError(f"{where}: {rc.dims} rotated dims do not fit a head of {dim}")
         return ChunkedAttentionConfig(heads, kv_heads, dim, vdim, scale, chunk, rc)
 
     def to_dict(self) -> dict:
-        return {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale,
-                "mask": {"size": self.chunk}, "rot": self.rot.to_dict()}
+        out = {"heads": self.heads, "kv_heads": self.kv_heads, "dim": self.dim, "vdim": self.vdim, "scale": self.scale}
+        if self.chunk:
+            out["mask"] = {"size": self.chunk}
+        if self.rot is not None:
+            out["rot"] = self.rot.to_dict()
+        return out
 
 
 @dataclass(frozen=True)

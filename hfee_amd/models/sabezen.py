@@ -23,8 +23,10 @@ from ..config.specs import (EmbeddingSpec, FeedForwardSpec, LayerSpec, MixerSpec
 
 def _mixer(cfg: SabezenConfig, m) -> MixerSpec:
     if isinstance(m, ChunkedAttentionConfig):
-        position = PositionSpec("rope", params(head_dim=m.dim, rotary_dim=m.rot.dims, theta=m.rot.base, scaling=None,
-                                               pairing="half"))
+        position = None
+        if m.rot is not None:
+            position = PositionSpec("rope", params(head_dim=m.dim, rotary_dim=m.rot.dims, theta=m.rot.base, scaling=None,
+                                                   pairing="half"))
         return MixerSpec("mixed_attention", params(
             hidden=cfg.width, num_heads=m.heads, num_kv_heads=m.kv_heads, dim=m.dim, scale=m.scale, chunk=m.chunk,
             sink="zero", head_mix=True, qk_norm="rms_after_rotation", norm_eps=cfg.norm_eps, values="keys",

@@ -57,14 +57,15 @@ def chunked_talking_attention(h, w, pre, m, eps):
     q = (h @ w[pre + "q"].T).view(T, H, D)
     k = (h @ w[pre + "k"].T).view(T, G, D)
     v = k
-    q = rms(rotate_half(q, pos, m["rot"]["dims"], m["rot"]["base"]), eps)
-    kr = rms(rotate_half(k, pos, m["rot"]["dims"], m["rot"]["base"]), eps)
+    rot = m.get("rot") or {"dims": 0, "base": 2.0}            # (no rotation named: none)
+    q = rms(rotate_half(q, pos, rot["dims"], rot["base"]), eps)
+    kr = rms(rotate_half(k, pos, rot["dims"], rot["base"]), eps)
     rep = H // G
     kh = kr.repeat_interleave(rep, dim=1)                                 # [T, H, D]
     vh = v.repeat_interleave(rep, dim=1)
     s = torch.einsum("ihd,jhd->hij", q, kh) * m["scale"]                  # [H, T, T]
     s = torch.einsum("hg,gij->hij", w[pre + "talk"].to(s.dtype), s)
-    size = m["mask"]["size"]
+    size = (m.get("mask") or {"size": T})["size"]             # (no mask named: every earlier position)
     seen = (pos[None, :] <= pos[:, None]) & ((pos[None, :] // size) == (pos[:, None] // size))
     e = torch.where(seen[None], torch.exp(s), torch.zeros_like(s))
     p = e / (1 + e.sum(-1, keepdim=True))

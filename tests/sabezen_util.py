@@ -76,6 +76,8 @@ CONFIGS = {"A": S_A, "B": S_B, "C": S_C, "D": S_D}
 # one mechanism each
 SINGLE = {
     "attention": config(50, 48, 1e-6, 2.0, [bare(attention(4, 2, 12, 6, 10, 0.4))]),
+    "attention without chunks or rotation": config(50, 64, 1e-6, 2.0, [bare(
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 4, "dim": 32, "scale": 0.2}})]),
     "delta": config(50, 48, 1e-6, 2.0, [bare(delta(4, 2, 8, 12, 3, 6, 6))]),
     "gla": config(50, 48, 1e-6, 2.0, [bare(gla(3, 8, 12, 5.0, 6))]),
     "dense": config(50, 48, 1e-6, 2.0, [dense(gla(1, 4, 4, 5.0, 2), 40)]),

@@ -35,6 +35,10 @@ def test_the_configuration_reads_ranks_from_the_tensors(tmp_path):
     bad["layers"][3]["mlp"]["router"]["top"] = 9
     with pytest.raises(ConfigError, match="experts"):
         config_from_dict(bad)
+    bare = json.loads(json.dumps(su.S_A))
+    del bare["layers"][0]["mixer"]["mask"], bare["layers"][0]["mixer"]["rot"]
+    plain = config_from_dict(bare).layers[0].mixer
+    assert plain.chunk == 0 and plain.rot is None and config_from_dict(config_from_dict(bare).to_dict()).layers[0].mixer == plain
     bad = json.loads(json.dumps(su.S_A))
     bad["layers"][2]["type"] = "window"
     with pytest.raises(ConfigError, match="unknown mixer"):
