@@ -460,6 +460,30 @@ def test_long_decoding(folders, dtype):
     compare(got, {("a", i): want[i] for i in range(29, 330)}, TOL[dtype], f"long decoding {dtype}")
 
 
+def test_grouped_experts_inside_replayed_decode_steps(tmp_path):
+    """Three requests decode side by side on a model of two experts, both for every token: more pairs than
+    experts, so the grouped kernels (their ordering on the device included) run inside the recorded graphs."""
+    from hfee_amd.trace_replay import Replayer
+    cj = su.config(70, 64, 1e-6, 2.0, [su.moe(su.gla(2, 16, 16, 6.0, 8), 32, 2, 2), su.moe(su.attention(4, 2, 32, 16, 24, 0.2), 64, 3, 2)])
+    folder = su.make_folder(tmp_path / "few", cj, seed=5, dtype="bfloat16")
+    reqs = tu.make_requests(70, [50, 47, 44], seed=1)
+    steps = [{"entries": [(rid, toks[:4], [3]) for rid, toks in reqs.items()], "end": []}]
+    for i in range(4, 44):
+        steps.append({"entries": [(rid, toks[i:i + 1], [0]) for rid, toks in reqs.items()], "end": []})
+    steps.append({"entries": [(rid, toks[44:], [len(toks) - 45]) for rid, toks in reqs.items() if len(toks) > 44],
+                  "end": list(reqs)})
+    rep = Replayer(folder, "bfloat16", 256, max_requests=4)
+    got = tu.run(rep, steps)
+    assert rep.engine.graph_replays > 30
+    want = {}
+    for rid, toks in reqs.items():
+        logits = plain_logits(folder, toks)
+        want.update({(rid, i): logits[i] for i in range(3, 44)})
+        if len(toks) > 44:
+            want[(rid, len(toks) - 1)] = logits[len(toks) - 1]
+    compare(got, want, TOL["bfloat16"], "grouped experts in graphs")
+
+
 def test_a_far_token_shows_through_the_states(folders):
     """Two sequences that differ in their first token only: hundreds of tokens later the recurrent layers
     still carry the difference (no attention layer could: the chunks are long past), and the engine's
