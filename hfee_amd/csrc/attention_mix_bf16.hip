@@ -1,15 +1,17 @@
 // Attention whose heads' scores are mixed before the softmax, on the matrix cores; bfloat16, compiled
-// for one number of heads H (HFEE_MIX_HEADS, a multiple of 4) and one head size D (HFEE_MIX_DIM, a
-// multiple of 32).  What is computed is what attention_mix.hip computes (keys of the query's chunk up to
+// for one number of heads H (HFEE_MIX_HEADS, a multiple of 4), of key heads G (HFEE_MIX_KV_HEADS) and one
+// head size D (HFEE_MIX_DIM, a multiple of 32).  What is computed is what attention_mix.hip computes (keys of the query's chunk up to
 // the query, scores of all heads mixed by a matrix, an optional sink, the keys as projected for values).
 //
 // A workgroup of four (or eight) waves takes an item: up to 16 consecutive rows of one sequence that lie in
 // one chunk, and all heads, a wave a quarter (an eighth) of them.  Keys come in tiles of 16 that start at multiples of 16 of
 // the sequence's positions (a tile lies in one page; keys before the chunk are masked), so what is added
 // in which order depends on positions only.  A tile's steps:
-//   1. raw scores: v_mfma_f32_16x16x32_bf16, the tile's keys as the first operand straight from the
-//      page, the rows' queries (held in registers for all tiles) as the second; lane l then holds, for
-//      row l % 16, the keys 4 (l / 16) .. + 3: sixteen bytes of raw[head][row][key] in LDS.
+//   0. everything the tile needs from memory is asked for at once: the keys of the wave's key heads (once a
+//      key head, whichever of the wave's heads read it), their value columns, the rows' queries.
+//   1. raw scores: v_mfma_f32_16x16x32_bf16, the tile's keys as the first operand, the rows' queries as
+//      the second; lane l then holds, for row l % 16, the keys 4 (l / 16) .. + 3: sixteen bytes of
+//      raw[head][row][key] in LDS.
 //   2. mixing on the vector units in float32: the wave's heads h, s_h = sum_g T[h][g] raw_g for the lane's
 //      row and four keys; T comes transposed ([g][h]) through scalar loads, the same for all lanes.
 //   3. the softmax's running maximum and sum for each (head, row), over the lane's four keys and the
@@ -24,19 +26,25 @@
 
 using namespace hfee;
 
-#ifndef HFEE_MIX_HEADS
-#error "compile with -DHFEE_MIX_HEADS=<heads> -DHFEE_MIX_DIM=<head size>"
+#if !defined(HFEE_MIX_HEADS) || !defined(HFEE_MIX_KV_HEADS) || !defined(HFEE_MIX_DIM)
+#error "compile with -DHFEE_MIX_HEADS=<heads> -DHFEE_MIX_KV_HEADS=<key heads> -DHFEE_MIX_DIM=<head size>"
 #endif
 
 namespace {
 
-constexpr int H = HFEE_MIX_HEADS, D = HFEE_MIX_DIM;
+constexpr int H = HFEE_MIX_HEADS, G = HFEE_MIX_KV_HEADS, D = HFEE_MIX_DIM, PER_KV = H / G;
+static_assert(H % G == 0, "heads are a multiple of key heads");
 // (what a wave keeps in registers for all tiles, its heads' queries and outputs, is 3/8 of a register a
 // head and dim: four waves where that fits their 512 registers, eight waves of half as many heads and
 // 256 registers beyond)
 constexpr int WAVES = H / 4 * D > 512 ? 8 : 4;
 constexpr int HW = H / WAVES, KS = D / 32, DB = D / 16, ROWS = 16, KEYS = 16;
 static_assert(H % WAVES == 0 && D % 32 == 0 && HW * D <= 512, "heads in fours or eights, head sizes in multiples of 32");
+// the most key heads that the consecutive heads of a wave read
+constexpr int NKV = (HW + PER_KV - 2) / PER_KV + 1 < G ? (HW + PER_KV - 2) / PER_KV + 1 : G;
+// value columns wait in registers from the tile's start where they fit beside the outputs (else they are
+// asked for head by head, behind the softmax)
+constexpr bool EARLY_VALUES = HW * D / 4 + NKV * D / 4 + 72 <= (WAVES == 8 ? 256 : 512);
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -65,15 +73,9 @@ __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
   const int lane = threadIdx.x & 63, r16 = lane & 15, kq = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int first = chunk > 0 ? p0 / chunk * chunk : 0, last = p0 + rows - 1;
-  const int per_kv = H / lay.kv_heads;
   const int my_row = r16 < rows ? r16 : rows - 1;
-
-  Operand8 qop[HW][KS];
-#pragma unroll
-  for (int hh = 0; hh < HW; ++hh)
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qop[hh][ks].u = *reinterpret_cast<const u32x4*>(q + (int64_t)(row0 + my_row) * ldq + (wave * HW + hh) * D + ks * 32 + kq * 8);
+  const int kv0 = wave * HW / PER_KV;                       // the first key head that this wave's heads read
+  const bf16_t* q_row = q + (int64_t)(row0 + my_row) * ldq + wave * HW * D + kq * 8;
 
   // this workgroup's share of the item's key tiles
   const int tile0 = first / KEYS, tiles = last / KEYS - tile0 + 1, share = (tiles + splits - 1) / splits;
@@ -93,17 +95,33 @@ __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
 
   for (int j0 = j_begin; j0 < j_end; j0 += KEYS) {
     const int page = bt[j0 >> lay.page_shift], slot0 = j0 & (lay.page_size - 1);
+    // 0. the tile's loads
+    Operand8 kop[NKV][KS];
+    Operand4 vop[EARLY_VALUES ? NKV : 1][DB];
+#pragma unroll
+    for (int kv = 0; kv < NKV; ++kv) {
+      const int kvh = min(kv0 + kv, G - 1);
+      const bf16_t* kr = cache + lay.key_offset(page, kvh, slot0 + r16, kq * 8);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kop[kv][ks].u = *reinterpret_cast<const u32x4*>(kr + ks * 32);
+      if constexpr (EARLY_VALUES) {
+        const bf16_t* vr = cache + lay.value_offset(page, kvh, slot0 + kq * 4, r16);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vop[kv][db].u = *reinterpret_cast<const u32x2*>(vr + (int64_t)db * 16 * lay.page_size);
+      }
+    }
     // 1. raw scores of the wave's heads
 #pragma unroll
     for (int hh = 0; hh < HW; ++hh) {
-      const int g = wave * HW + hh;
-      const bf16_t* kr = cache + lay.key_offset(page, g / per_kv, slot0 + r16, kq * 8);
+      const int g = wave * HW + hh, kv = g / PER_KV - kv0;
       f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        Operand8 kop;
-        kop.u = *reinterpret_cast<const u32x4*>(kr + ks * 32);
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop.v, qop[hh][ks].v, s, 0, 0, 0);
+        Operand8 qop;
+        qop.u = *reinterpret_cast<const u32x4*>(q_row + hh * D + ks * 32);
+#pragma unroll
+        for (int c = 0; c < NKV; ++c)        // (which of the wave's key heads: the same for all lanes)
+          if (c == kv) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[c][ks].v, qop.v, s, 0, 0, 0);
       }
       *reinterpret_cast<f32x4*>(&raw[g][r16][kq * 4]) = s * scale;
     }
@@ -114,7 +132,7 @@ __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
 #pragma unroll
       for (int hh = 0; hh < HW; ++hh) sc[hh] = f32x4{0.f, 0.f, 0.f, 0.f};
       const float* tw = mix_t + wave * HW;
-#pragma unroll 4
+#pragma unroll 8
       for (int g = 0; g < H; ++g) {
         const f32x4 r = *reinterpret_cast<const f32x4*>(&raw[g][r16][kq * 4]);
 #pragma unroll
@@ -129,41 +147,65 @@ __global__ __launch_bounds__(WAVES * 64) void mix_attend_bf16_kernel(
       for (int hh = 0; hh < HW; ++hh) sc[hh] = *reinterpret_cast<const f32x4*>(&raw[wave * HW + hh][r16][kq * 4]);
     }
     __syncthreads();
-    // 3. and 4. head by head
+    // 3. the running softmax of all the wave's heads (their exchanges between lanes side by side)
+    bool seen[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = j0 + kq * 4 + i;
+      seen[i] = j >= first && j <= p0 + r16 && r16 < rows;
+    }
+    float tmax[HW], psum[HW], shrink[HW];
+    Operand4 pop[HW];
 #pragma unroll
     for (int hh = 0; hh < HW; ++hh) {
-      const int kvh = (wave * HW + hh) / per_kv;
-      float tmax = -INFINITY;
-      bool seen[4];
+      tmax[hh] = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int j = j0 + kq * 4 + i;
-        seen[i] = j >= first && j <= p0 + r16 && r16 < rows;
-        if (seen[i]) tmax = fmaxf(tmax, sc[hh][i]);
-      }
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-      const float m_new = fmaxf(m[hh], tmax);
-      float p[4], psum = 0.f;
+      for (int i = 0; i < 4; ++i)
+        if (seen[i]) tmax[hh] = fmaxf(tmax[hh], sc[hh][i]);
+    }
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) tmax[hh] = fmaxf(tmax[hh], __shfl_xor(tmax[hh], 16, kWave));
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) tmax[hh] = fmaxf(tmax[hh], __shfl_xor(tmax[hh], 32, kWave));
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      const float m_new = fmaxf(m[hh], tmax[hh]);
+      float p[4];
+      psum[hh] = 0.f;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         p[i] = seen[i] ? expf(sc[hh][i] - m_new) : 0.f;
-        psum += p[i];
+        psum[hh] += p[i];
       }
-      psum += __shfl_xor(psum, 16, kWave);
-      psum += __shfl_xor(psum, 32, kWave);
-      const float shrink = m[hh] == -INFINITY ? 0.f : expf(m[hh] - m_new);      // (m_new is finite wherever m is)
-      l[hh] = fmaf(l[hh], shrink, psum);
+      shrink[hh] = m[hh] == -INFINITY ? 0.f : expf(m[hh] - m_new);      // (m_new is finite wherever m is)
       m[hh] = m_new;
-      Operand4 pop;
-      pop.u = u32x2{(uint32_t)float_to_bf16(p[0]) | ((uint32_t)float_to_bf16(p[1]) << 16),
-                    (uint32_t)float_to_bf16(p[2]) | ((uint32_t)float_to_bf16(p[3]) << 16)};
-      const bf16_t* vr = cache + lay.value_offset(page, kvh, slot0 + kq * 4, r16);
+      pop[hh].u = u32x2{(uint32_t)float_to_bf16(p[0]) | ((uint32_t)float_to_bf16(p[1]) << 16),
+                        (uint32_t)float_to_bf16(p[2]) | ((uint32_t)float_to_bf16(p[3]) << 16)};
+    }
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        Operand4 vop;
-        vop.u = *reinterpret_cast<const u32x2*>(vr + (int64_t)db * 16 * lay.page_size);
-        o[hh][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop.v, pop.v, o[hh][db] * shrink, 0, 0, 0);
+    for (int hh = 0; hh < HW; ++hh) psum[hh] += __shfl_xor(psum[hh], 16, kWave);
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) psum[hh] += __shfl_xor(psum[hh], 32, kWave);
+    // 4. the weighted values
+#pragma unroll
+    for (int hh = 0; hh < HW; ++hh) {
+      l[hh] = fmaf(l[hh], shrink[hh], psum[hh]);
+      const int kv = (wave * HW + hh) / PER_KV - kv0;
+      if constexpr (EARLY_VALUES) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const f32x4 before = o[hh][db] * shrink[hh];
+#pragma unroll
+          for (int c = 0; c < NKV; ++c)
+            if (c == kv) o[hh][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop[c][db].v, pop[hh].v, before, 0, 0, 0);
+        }
+      } else {
+        const bf16_t* vr = cache + lay.value_offset(page, kv0 + kv, slot0 + kq * 4, r16);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) vop[0][db].u = *reinterpret_cast<const u32x2*>(vr + (int64_t)db * 16 * lay.page_size);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+          o[hh][db] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vop[0][db].v, pop[hh].v, o[hh][db] * shrink[hh], 0, 0, 0);
       }
     }
   }
@@ -226,6 +268,7 @@ __global__ __launch_bounds__(256) void mix_join_kernel(bf16_t* __restrict__ out,
 HFEE_DEFINE_LAST_ERROR
 
 HFEE_API int hfee_attention_mix_bf16_heads() { return H; }
+HFEE_API int hfee_attention_mix_bf16_kv_heads() { return G; }
 HFEE_API int hfee_attention_mix_bf16_dim() { return D; }
 
 // items: int32 [count][4] on the device: first row, rows (1..16), first position, block-table row; the rows
@@ -239,7 +282,7 @@ HFEE_API int hfee_attention_mix_bf16(void* out, int64_t ld_out, const void* q, i
                                      hipStream_t stream) {
   HFEE_REQUIRE(count >= 0, "attention_mix_bf16: bad item count");
   if (count == 0) return 0;
-  HFEE_REQUIRE(kv_heads > 0 && H % kv_heads == 0, "attention_mix_bf16: %d heads are not a multiple of %d kv heads", H, kv_heads);
+  HFEE_REQUIRE(kv_heads == G, "attention_mix_bf16: compiled for %d key heads, called with %d", G, kv_heads);
   HFEE_REQUIRE(chunk >= 0 && sink_mode >= 0 && sink_mode <= 2 && (sink_mode != 2 || sinks != nullptr),
                "attention_mix_bf16: bad chunk or sink");
   HFEE_REQUIRE(ldq >= (int64_t)H * D && ld_out >= (int64_t)H * D && ldq % 8 == 0 && ld_out % 4 == 0 &&

@@ -6,8 +6,8 @@ Two kinds of library:
     size each, on demand (a model compiles only the head size it has);
   * `attention_kv_bf16_k<Dk>_v<Dv>`: the matrix-core attention for keys and values of
     different sizes, compiled per pair of sizes, on demand;
-  * `attention_mix_bf16_h<H>_d<D>`: the matrix-core attention whose heads' scores are mixed,
-    compiled per number of heads and head size, on demand.
+  * `attention_mix_bf16_h<H>_g<G>_d<D>`: the matrix-core attention whose heads' scores are mixed,
+    compiled per number of heads, of key heads and head size, on demand.
 Libraries are built in-tree (hfee_amd/_lib); if that folder cannot be written, in a
 per-user folder under the system's temporary directory; $HFEE_BUILD_DIR, if set, comes
 before both.  A library is rebuilt when its sources or flags no longer match the stamp
@@ -41,9 +41,9 @@ ATTENTION_SOURCE = "attention_bf16.hip"
 HEAD_DIMS = tuple(range(16, 257, 16))
 ATTENTION_KV_SOURCE = "attention_kv_bf16.hip"      # compiled per (key size, value size)
 ATTENTION_KV_MOST = (1024, 512)
-ATTENTION_MIX_SOURCE = "attention_mix_bf16.hip"    # compiled per (heads, head size)
-# the pairs that `build_all` compiles: those of the tests and of bench.py's comparison
-ATTENTION_MIX_SIZES = ((4, 32), (8, 32), (8, 64), (16, 128), (32, 128))
+ATTENTION_MIX_SOURCE = "attention_mix_bf16.hip"    # compiled per (heads, key heads, head size)
+# the sizes that `build_all` compiles: those of the tests and of bench.py's comparison
+ATTENTION_MIX_SIZES = ((4, 2, 32), (4, 4, 32), (8, 2, 32), (8, 8, 32), (8, 2, 64), (16, 4, 128), (32, 8, 128))
 
 
 def attention_mix_fits(heads: int, dim: int) -> bool:
@@ -132,12 +132,14 @@ def library_spec(name: str):
         return [ATTENTION_KV_SOURCE], [f"-DHFEE_DK={dk}", f"-DHFEE_DV={dv}"]
     if name.startswith("attention_mix_bf16_h"):
         try:
-            heads, dim = (int(n) for n in name[len("attention_mix_bf16_h"):].split("_d"))
+            heads, rest = name[len("attention_mix_bf16_h"):].split("_g")
+            kv_heads, dim = rest.split("_d")
+            heads, kv_heads, dim = int(heads), int(kv_heads), int(dim)
         except ValueError:
             raise BuildError(f"unknown kernel library {name!r}") from None
-        if not attention_mix_fits(heads, dim):
-            raise BuildError(f"the matrix-core attention with mixed heads does not take {heads} heads of {dim}")
-        return [ATTENTION_MIX_SOURCE], [f"-DHFEE_MIX_HEADS={heads}", f"-DHFEE_MIX_DIM={dim}"]
+        if not attention_mix_fits(heads, dim) or kv_heads < 1 or heads % kv_heads:
+            raise BuildError(f"the matrix-core attention with mixed heads does not take {heads} heads on {kv_heads} of {dim}")
+        return [ATTENTION_MIX_SOURCE], [f"-DHFEE_MIX_HEADS={heads}", f"-DHFEE_MIX_KV_HEADS={kv_heads}", f"-DHFEE_MIX_DIM={dim}"]
     raise BuildError(f"unknown kernel library {name!r}")
 
 
@@ -217,7 +219,7 @@ def build_all(head_dims=HEAD_DIMS, force: bool = True, kv_sizes=ATTENTION_KV_SIZ
     out = [build_library("core", force=force)]
     # the attention libraries are independent: build them side by side
     names = [f"attention_bf16_hd{hd}" for hd in head_dims] + [f"attention_kv_bf16_k{dk}_v{dv}" for dk, dv in kv_sizes]
-    names += [f"attention_mix_bf16_h{h}_d{d}" for h, d in mix_sizes]
+    names += [f"attention_mix_bf16_h{h}_g{g}_d{d}" for h, g, d in mix_sizes]
     errors = []
 
     def work(n):

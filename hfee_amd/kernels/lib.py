@@ -76,6 +76,7 @@ _ATTENTION_KV_SIGNATURES = {
 
 _ATTENTION_MIX_SIGNATURES = {
     "hfee_attention_mix_bf16_heads": [],
+    "hfee_attention_mix_bf16_kv_heads": [],
     "hfee_attention_mix_bf16_dim": [],
     "hfee_attention_mix_bf16": [P, L, P, L, P, P, I, P, I, I, I, F, P, I, I, P, I, P, L, P],
 }
@@ -155,8 +156,8 @@ def attention_kv_bf16(dk: int, dv: int) -> Library:
     return load(f"attention_kv_bf16_k{dk}_v{dv}")
 
 
-def attention_mix_bf16(heads: int, dim: int) -> Library:
-    """The matrix-core attention with mixed heads for this number of heads and head size."""
-    if not build.attention_mix_fits(heads, dim):
-        raise KernelError(f"the matrix-core attention with mixed heads does not take {heads} heads of {dim}")
-    return load(f"attention_mix_bf16_h{heads}_d{dim}")
+def attention_mix_bf16(heads: int, kv_heads: int, dim: int) -> Library:
+    """The matrix-core attention with mixed heads for these numbers of heads and key heads and this head size."""
+    if not build.attention_mix_fits(heads, dim) or kv_heads < 1 or heads % kv_heads:
+        raise KernelError(f"the matrix-core attention with mixed heads does not take {heads} heads on {kv_heads} of {dim}")
+    return load(f"attention_mix_bf16_h{heads}_g{kv_heads}_d{dim}")

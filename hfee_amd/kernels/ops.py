@@ -1122,7 +1122,7 @@ def attention_mix_bf16(out, q, cache_layer, items, block_tables, num_heads: int,
         _check(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == num_heads,
                "attention_mix: sinks must be float32 [heads]")
         sinks, mode = sink, 2
-    lib.attention_mix_bf16(num_heads, dim).call(
+    lib.attention_mix_bf16(num_heads, kv_heads, dim).call(
         "hfee_attention_mix_bf16", _ptr(out), ldo, _ptr(q), ldq, _ptr(cache_layer), _ptr(items), items.shape[0],
         _ptr(block_tables), block_tables.stride(0), kv_heads, page_size, float(scale), _ptr(mix_t), int(chunk), mode,
         _ptr(sinks), int(splits), _ptr(partial), 0 if partial is None else partial.numel(), _stream())

@@ -28,7 +28,7 @@ from ..weights.spec import TensorSpec
 from .base import LazyNorm, Mixer, lookup, register_mixer
 from .kv_attention import product, tiles_of
 
-_WORKGROUPS_WANTED = 512        # items split their keys until about this many workgroups run
+_WORKGROUPS_WANTED = 256        # items split their keys until about this many workgroups run (one a CU)
 _MOST_SPLITS = 8
 _PARTIAL_LIMIT = 64 << 20       # float32 words of the splits' parts
 _LAYOUT = "by key head: the keys as scored by slot, then the keys as projected by dimension"
